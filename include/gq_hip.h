@@ -1,0 +1,137 @@
+/*
+ * libgq_hip -- 4-bit group-quantized weight decompression and fused dequant-matmul
+ * for AMD MI355X (gfx950).  C ABI: plain pointers and sizes, no C++ or torch types.
+ *
+ * This library stands where the reference's pybind11 extension
+ * `group_quantize_decompress_binding` stands
+ * (popxl_addons/ops/group_quantize_decompress/group_quantize_decompress_binding.cpp:39-55):
+ * the Python wrappers of the reference call `GroupQuantizeDecompressOp.createOpInGraph`
+ * there; here they call the functions below with device pointers.
+ *
+ * Conventions
+ *   - Every data pointer is a DEVICE pointer owned by the caller.  binary16 values are
+ *     passed as their 16-bit patterns (`uint16_t`).
+ *   - Work is enqueued on `stream` (a `hipStream_t` passed as `void*`; NULL = the null
+ *     stream) and the call returns without synchronising.
+ *   - Return value: 0 on success; a negative GQ_ERR_* code when an argument is rejected
+ *     (nothing was launched); a positive value is a `hipError_t` from the runtime.
+ *     `gq_last_error()` returns a thread-local, human-readable description of the last
+ *     non-zero return on the calling thread.
+ *   - Functions are re-entrant and keep no per-call state; the split-K workspace of the
+ *     matmul entry points is per device and protected per stream by stream order only:
+ *     two matmul calls running concurrently on different streams of one device must not
+ *     both use split-K shapes (see gq_linear_f16).
+ *
+ * Packed layout (group_quantize_decompress.py:127-135, group_quantize_decompress_codelet.cpp:11-14)
+ *   packed[r][g][i] is a little-endian uint16 holding four 4-bit codes, most significant
+ *   nibble first: element 4*i+j of group g of row r is (packed[r][g][i] >> (12 - 4*j)) & 15.
+ *   value = f16( f16(code * scale[r][g]) + bias[r][g] )   -- two roundings, never an fma.
+ */
+#ifndef GQ_HIP_H
+#define GQ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GQ_ABI_VERSION 1
+
+#define GQ_OK 0
+#define GQ_ERR_NULL_POINTER (-1) /* a required pointer is NULL */
+#define GQ_ERR_BAD_SHAPE (-2)    /* a size is negative, or sizes are inconsistent */
+#define GQ_ERR_MISALIGNED (-3)   /* a pointer is not aligned to its element size */
+#define GQ_ERR_UNSUPPORTED (-4)  /* well-formed, but outside what the kernels cover */
+#define GQ_ERR_NO_DEVICE (-5)    /* no usable gfx950 device / code object */
+
+/* ABI version of the loaded library (GQ_ABI_VERSION it was built with). */
+int gq_abi_version(void);
+
+/* Thread-local description of the last failing call on this thread ("" if none). */
+const char *gq_last_error(void);
+
+/* Tuning/diagnostic switches, by name.  Unknown names return GQ_ERR_UNSUPPORTED.
+ *   "decompress_variant"  kernel flavour of gq_decompress_f16 (0 = default)
+ *   "gemv_variant"        kernel flavour of gq_gemv_f16       (0 = default)
+ *   "gemm_variant"        kernel flavour of gq_gemm_f16       (0 = default) */
+int gq_set_option(const char *name, int64_t value);
+
+/*
+ * Standalone decompress.  Replaces the device op created by
+ * group_quantize_decompress() (group_quantize_decompress.py:78-86), whose lowering is
+ * GroupQuantizeDecompressOpx::grow (group_quantize_decompressx.cpp:121-135: unpack vertex,
+ * then scale and bias as a second pass) with shape rules of
+ * GroupQuantizeDecompressOp::setup (group_quantize_decompress.cpp:35-77).
+ *
+ *   packed [rows, n_groups, n_ids] uint16      scale, bias [rows, n_groups] binary16
+ *   out    [rows, n_groups * n_ids * 4] binary16, row-major, bit-exact to
+ *          group_quantize_decompress_numpy (group_quantize_decompress.py:95-141).
+ * Zero-sized problems succeed without a launch.
+ */
+int gq_decompress_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                      uint16_t *out, int64_t rows, int64_t n_groups, int64_t n_ids, void *stream);
+
+/*
+ * Same values written transposed: out_t [n_groups * n_ids * 4, rows].  This is the
+ * `dim=0` result of group_quantize_decompress (group_quantize_decompress.py:87-91 moves
+ * the decompressed axis to `dim`), materialised instead of returned as a strided view.
+ */
+int gq_decompress_f16_transposed(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                                 uint16_t *out_t, int64_t rows, int64_t n_groups, int64_t n_ids,
+                                 void *stream);
+
+/*
+ * Fused decompress + matmul, groups along the input (K) axis: the computation of
+ * LinearGQ.build with dim=0 (popxl_addons/layers/linear_gq.py:99-109):
+ *   w = decompress(packed, scale, bias)      [n_out, k_in]
+ *   y[m][n] = sum_k x[m][k] * w[n][k] (+ out_bias[n])
+ * without writing w to memory.
+ *
+ *   x        [m_rows, k_in] binary16             y [m_rows, n_out] binary16
+ *   packed   [n_out, k_in / group_size, group_size / 4] uint16
+ *   scale, bias [n_out, k_in / group_size] binary16
+ *   out_bias [n_out] binary16 or NULL
+ * Accumulation is binary32; the result is within 1e-2 (max-abs normalised) of a binary32
+ * matmul over the bit-exact decompressed weight.
+ *
+ * gq_gemv_f16  decode-sized batches, 1 <= m_rows <= 16.
+ * gq_gemm_f16  prefill-sized batches (any m_rows >= 1; built for m_rows >= 16).
+ * gq_linear_f16 picks between them by m_rows; it is what the LinearGQ wrapper calls.
+ *
+ * Shapes with k_in > 4096 are split along K over several workgroups that meet in a
+ * per-device workspace owned by the library: calls on ONE stream are ordered and safe;
+ * concurrent calls of such shapes on different streams of the same device are not.
+ * Requirements: group_size % 4 == 0, k_in % group_size == 0.
+ */
+int gq_gemv_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                int64_t k_in, int64_t group_size, void *stream);
+
+int gq_gemm_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                int64_t k_in, int64_t group_size, void *stream);
+
+int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                  int64_t k_in, int64_t group_size, void *stream);
+
+/*
+ * Device-side compress for binary16 input: bit-identical packed/scale/bias to
+ * group_quantize_compress_numpy on a float16 array (group_quantize_decompress.py:178-196)
+ * wherever that function is defined (every group has max > min; all values finite).
+ * A constant group yields scale 0, codes 0, bias = the constant.
+ *
+ *   t [rows, n_groups * group_size] binary16  ->  packed [rows, n_groups, group_size/4],
+ *   scale, bias [rows, n_groups].
+ * `nonfinite_flag` (device int32, may be NULL) is set to 1 when any input is Inf/NaN
+ * (the reference raises ValueError there, :182-183); outputs are then unspecified.
+ */
+int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,
+                    int32_t *nonfinite_flag, int64_t rows, int64_t n_groups, int64_t group_size,
+                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GQ_HIP_H */

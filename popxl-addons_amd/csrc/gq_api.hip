@@ -1,0 +1,165 @@
+// C-ABI layer of libgq_hip: argument validation, error text, dispatch to the launchers.
+// Shape rules follow GroupQuantizeDecompressOp::setup (group_quantize_decompress.cpp:35-77)
+// and LinearGQ.build (popxl_addons/layers/linear_gq.py:58-110).
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "gq_common.h"
+
+namespace gq {
+
+namespace {
+thread_local char g_error[512] = "";
+std::atomic<int> g_decompress_variant{0}, g_gemv_variant{0}, g_gemm_variant{0};
+}  // namespace
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return GQ_OK;
+  return fail((int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+int option_decompress_variant() { return g_decompress_variant.load(std::memory_order_relaxed); }
+int option_gemv_variant() { return g_gemv_variant.load(std::memory_order_relaxed); }
+int option_gemm_variant() { return g_gemm_variant.load(std::memory_order_relaxed); }
+
+namespace {
+
+bool misaligned(const void *p, size_t a) { return ((uintptr_t)p % a) != 0; }
+
+int check_linear_args(const char *who, const uint16_t *x, int64_t m_rows, const uint16_t *packed,
+                      const uint16_t *scale, const uint16_t *bias, const uint16_t *out_bias, uint16_t *y,
+                      int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (m_rows < 0 || n_out < 0 || k_in < 0)
+    return fail(GQ_ERR_BAD_SHAPE, "%s: negative size (m_rows=%lld n_out=%lld k_in=%lld)", who,
+                (long long)m_rows, (long long)n_out, (long long)k_in);
+  if (group_size <= 0 || group_size % 4 != 0)
+    return fail(GQ_ERR_BAD_SHAPE, "%s: group_size=%lld must be a positive multiple of 4", who,
+                (long long)group_size);
+  if (k_in % group_size != 0)
+    return fail(GQ_ERR_BAD_SHAPE, "%s: k_in=%lld is not a multiple of group_size=%lld", who, (long long)k_in,
+                (long long)group_size);
+  if (m_rows == 0 || n_out == 0) return GQ_OK;
+  if (!y) return fail(GQ_ERR_NULL_POINTER, "%s: y is NULL", who);
+  if (k_in > 0 && (!x || !packed || !scale || !bias))
+    return fail(GQ_ERR_NULL_POINTER, "%s: x/packed/scale/bias must not be NULL", who);
+  if (misaligned(x, 2) || misaligned(packed, 2) || misaligned(scale, 2) || misaligned(bias, 2) ||
+      misaligned(out_bias, 2) || misaligned(y, 2))
+    return fail(GQ_ERR_MISALIGNED, "%s: pointers must be 2-byte aligned", who);
+  if (m_rows > (int64_t)1 << 30 || n_out > (int64_t)1 << 30 || k_in > (int64_t)1 << 30)
+    return fail(GQ_ERR_UNSUPPORTED, "%s: a dimension exceeds 2^30", who);
+  return 1;  // proceed
+}
+
+int decompress_common(const char *who, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                      uint16_t *out, int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed,
+                      void *stream) {
+  if (rows < 0 || n_groups < 0 || n_ids < 0)
+    return fail(GQ_ERR_BAD_SHAPE, "%s: negative size (rows=%lld n_groups=%lld n_ids=%lld)", who,
+                (long long)rows, (long long)n_groups, (long long)n_ids);
+  if (rows == 0 || n_groups == 0 || n_ids == 0) return GQ_OK;
+  if (!packed || !scale || !bias || !out) return fail(GQ_ERR_NULL_POINTER, "%s: NULL pointer argument", who);
+  if (misaligned(packed, 2) || misaligned(scale, 2) || misaligned(bias, 2) || misaligned(out, 2))
+    return fail(GQ_ERR_MISALIGNED, "%s: pointers must be 2-byte aligned", who);
+  if (rows > ((int64_t)1 << 40) / n_groups / n_ids)
+    return fail(GQ_ERR_UNSUPPORTED, "%s: more than 2^40 packed words", who);
+  return launch_decompress(packed, scale, bias, out, rows, n_groups, n_ids, transposed, (hipStream_t)stream);
+}
+
+}  // namespace
+}  // namespace gq
+
+extern "C" {
+
+int gq_abi_version(void) { return GQ_ABI_VERSION; }
+
+const char *gq_last_error(void) { return gq::g_error; }
+
+int gq_set_option(const char *name, int64_t value) {
+  if (!name) return gq::fail(GQ_ERR_NULL_POINTER, "gq_set_option: name is NULL");
+  if (!strcmp(name, "decompress_variant")) gq::g_decompress_variant = (int)value;
+  else if (!strcmp(name, "gemv_variant")) gq::g_gemv_variant = (int)value;
+  else if (!strcmp(name, "gemm_variant")) gq::g_gemm_variant = (int)value;
+  else return gq::fail(GQ_ERR_UNSUPPORTED, "gq_set_option: unknown option '%s'", name);
+  return GQ_OK;
+}
+
+int gq_decompress_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
+                      int64_t rows, int64_t n_groups, int64_t n_ids, void *stream) {
+  return gq::decompress_common("gq_decompress_f16", packed, scale, bias, out, rows, n_groups, n_ids, false,
+                               stream);
+}
+
+int gq_decompress_f16_transposed(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                                 uint16_t *out_t, int64_t rows, int64_t n_groups, int64_t n_ids,
+                                 void *stream) {
+  return gq::decompress_common("gq_decompress_f16_transposed", packed, scale, bias, out_t, rows, n_groups,
+                               n_ids, true, stream);
+}
+
+int gq_gemv_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                int64_t group_size, void *stream) {
+  const int rc = gq::check_linear_args("gq_gemv_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
+                                       k_in, group_size);
+  if (rc <= 0) return rc;
+  if (m_rows > 16)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_f16: m_rows=%lld exceeds 16; use gq_gemm_f16",
+                    (long long)m_rows);
+  return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+                         (hipStream_t)stream);
+}
+
+int gq_gemm_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                int64_t group_size, void *stream) {
+  const int rc = gq::check_linear_args("gq_gemm_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
+                                       k_in, group_size);
+  if (rc <= 0) return rc;
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+                         (hipStream_t)stream);
+}
+
+int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                  int64_t group_size, void *stream) {
+  const int rc = gq::check_linear_args("gq_linear_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
+                                       k_in, group_size);
+  if (rc <= 0) return rc;
+  if (m_rows <= 16)
+    return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+                           (hipStream_t)stream);
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+                         (hipStream_t)stream);
+}
+
+int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,
+                    int32_t *nonfinite_flag, int64_t rows, int64_t n_groups, int64_t group_size,
+                    void *stream) {
+  if (rows < 0 || n_groups < 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_compress_f16: negative size");
+  if (group_size <= 0 || group_size % 4 != 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_compress_f16: group_size=%lld must be a positive multiple of 4",
+                    (long long)group_size);
+  if (rows == 0 || n_groups == 0) return GQ_OK;
+  if (!t || !packed || !scale || !bias) return gq::fail(GQ_ERR_NULL_POINTER, "gq_compress_f16: NULL pointer argument");
+  if (gq::misaligned(t, 2) || gq::misaligned(packed, 2) || gq::misaligned(scale, 2) ||
+      gq::misaligned(bias, 2) || gq::misaligned(nonfinite_flag, 4))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_compress_f16: misaligned pointer");
+  if (rows > ((int64_t)1 << 40) / n_groups / group_size)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_compress_f16: more than 2^40 elements");
+  return gq::launch_compress(t, packed, scale, bias, nonfinite_flag, rows, n_groups, group_size,
+                             (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,40 @@
+// Internal helpers shared by the gfx950 kernels and the C-ABI layer of libgq_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gq_hip.h"
+
+namespace gq {
+
+// Records a message for gq_last_error() on the calling thread and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// Maps the runtime's last launch error (if any) to a return code, recording its text.
+int check_launch(const char *what);
+
+int option_decompress_variant();
+int option_gemv_variant();
+int option_gemm_variant();
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+// Launchers implemented next to their kernels.
+int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
+                      int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed, hipStream_t stream);
+int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                int64_t group_size, hipStream_t stream);
+int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                int64_t group_size, hipStream_t stream);
+int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
+                    int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
+
+}  // namespace gq

@@ -1,0 +1,214 @@
+// Standalone int4 -> fp16 group-quantization decompress for gfx950.
+//
+// Replaces the two device passes of the reference lowering
+// (group_quantize_decompressx.cpp:51-109: unpack vertex, then popops::map(_1*_2+_3))
+// with one pass.  HBM-bound: per element 0.5 B of codes + 4/group_size B of scale/bias are
+// read and 2 B are written.
+//
+// Numerics (group_quantize_decompress.py:133-134): value = f16(f16(code * scale) + bias).
+// This translation unit is compiled with -ffp-contract=off so the multiply and the add
+// stay two separately rounded packed-fp16 instructions; the build checks the ISA for that.
+#include "gq_common.h"
+
+namespace gq {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+__device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
+
+// One 32-bit word = two little-endian uint16 = eight codes.  Memory order of the results:
+// word bits 15:12, 11:8, 7:4, 3:0, then 31:28, 27:24, 23:20, 19:16 (most significant
+// nibble of each uint16 first, group_quantize_decompress.py:130).
+// Codes are made exact in fp16 by or-ing the nibble into the mantissa of 1024.0 (0x6400)
+// and subtracting 1024; each step handles the pair (element j, element j + 4).
+__device__ __forceinline__ uint4_t expand_word(uint32_t w, half2_t s2, half2_t b2) {
+  const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+  half2_t r[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t pair = ((w >> (12 - 4 * j)) & 0x000F000Fu) | 0x64006400u;
+    const half2_t code = as_half2(pair) - k1024;  // exact
+    const half2_t prod = code * s2;               // rounded to fp16
+    r[j] = prod + b2;                             // rounded to fp16 (no fma: contraction is off)
+  }
+  // r[j] = (element j, element j + 4)  ->  dwords (0,1) (2,3) (4,5) (6,7)
+  uint4_t o;
+  o.x = __builtin_amdgcn_perm(as_u32(r[1]), as_u32(r[0]), 0x05040100u);
+  o.y = __builtin_amdgcn_perm(as_u32(r[3]), as_u32(r[2]), 0x05040100u);
+  o.z = __builtin_amdgcn_perm(as_u32(r[1]), as_u32(r[0]), 0x07060302u);
+  o.w = __builtin_amdgcn_perm(as_u32(r[3]), as_u32(r[2]), 0x07060302u);
+  return o;
+}
+
+template <bool NT>
+__device__ __forceinline__ void store16(uint4_t *p, uint4_t v) {
+  if (NT)
+    __builtin_nontemporal_store(v, p);
+  else
+    *p = v;
+}
+
+template <typename T, bool NT>
+__device__ __forceinline__ T load_packed(const T *p) {
+  if (NT) return __builtin_nontemporal_load(p);
+  return *p;
+}
+
+// Fast path.  One work item = WORDS consecutive 32-bit words of the flattened packed tensor
+// (WORDS in {1, 2, 4}: a 4/8/16-byte load) -> WORDS 16-byte stores.  All words of an item
+// lie in one group (the launcher guarantees WORDS divides the words per group), so an item
+// needs one (scale, bias) pair.  Items are dealt to lanes so that consecutive lanes take
+// consecutive items: loads and stores of a wave are contiguous.
+template <int WORDS, int UNROLL, bool NT>
+__global__ __launch_bounds__(kThreads) void decompress_kernel(const uint32_t *__restrict__ packed,
+                                                              const half_t *__restrict__ scale,
+                                                              const half_t *__restrict__ bias,
+                                                              uint4_t *__restrict__ out, int64_t n_items,
+                                                              int items_per_group_shift,
+                                                              uint32_t items_per_group) {
+  typedef uint32_t vec_t __attribute__((ext_vector_type(WORDS)));
+  const int64_t base = (int64_t)blockIdx.x * (kThreads * UNROLL) + threadIdx.x;
+  vec_t w[UNROLL];
+  half_t s[UNROLL], b[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t item = base + (int64_t)u * kThreads;
+    if (item < n_items) {
+      w[u] = load_packed<vec_t, NT>(reinterpret_cast<const vec_t *>(packed) + item);
+      const int64_t group =
+          items_per_group_shift >= 0 ? (item >> items_per_group_shift) : (item / items_per_group);
+      s[u] = scale[group];
+      b[u] = bias[group];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int64_t item = base + (int64_t)u * kThreads;
+    if (item < n_items) {
+      const half2_t s2 = {s[u], s[u]}, b2 = {b[u], b[u]};
+      uint4_t *dst = out + item * WORDS;
+#pragma unroll
+      for (int k = 0; k < WORDS; ++k) store16<NT>(dst + k, expand_word(w[u][k], s2, b2));
+    }
+  }
+}
+
+// Any shape and any 2-byte alignment: one uint16 (four codes) per lane.
+__global__ __launch_bounds__(kThreads) void decompress_scalar_kernel(const uint16_t *__restrict__ packed,
+                                                                     const half_t *__restrict__ scale,
+                                                                     const half_t *__restrict__ bias,
+                                                                     half_t *__restrict__ out, int64_t n_words,
+                                                                     int64_t n_ids) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n_words) return;
+  const uint32_t w = packed[i];
+  const int64_t group = i / n_ids;
+  const half_t s = scale[group], b = bias[group];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const half_t code = (half_t)(float)((w >> (12 - 4 * j)) & 15u);
+    const half_t prod = code * s;
+    out[i * 4 + j] = prod + b;
+  }
+}
+
+// Transposed result out_t[c][r] (c = column of the decompressed row).  A workgroup expands a
+// tile of 64 rows x 16 uint16 (64 columns) into LDS and writes it out with rows contiguous.
+constexpr int kTileRows = 64, kTileWords = 16, kTileCols = kTileWords * 4;
+__global__ __launch_bounds__(kThreads) void decompress_transposed_kernel(
+    const uint16_t *__restrict__ packed, const half_t *__restrict__ scale, const half_t *__restrict__ bias,
+    half_t *__restrict__ out_t, int64_t rows, int64_t words_per_row, int64_t n_ids) {
+  __shared__ half_t tile[kTileCols][kTileRows + 2];
+  const int64_t row0 = (int64_t)blockIdx.y * kTileRows, word0 = (int64_t)blockIdx.x * kTileWords;
+  const int64_t n_groups = words_per_row / n_ids;
+  for (int t = threadIdx.x; t < kTileRows * kTileWords; t += kThreads) {
+    const int r = t / kTileWords, wi = t % kTileWords;
+    const int64_t row = row0 + r, word = word0 + wi;
+    if (row < rows && word < words_per_row) {
+      const uint32_t w = packed[row * words_per_row + word];
+      const int64_t group = row * n_groups + word / n_ids;
+      const half_t s = scale[group], b = bias[group];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const half_t code = (half_t)(float)((w >> (12 - 4 * j)) & 15u);
+        const half_t prod = code * s;
+        tile[wi * 4 + j][r] = prod + b;
+      }
+    }
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < kTileCols * kTileRows; t += kThreads) {
+    const int c = t / kTileRows, r = t % kTileRows;
+    const int64_t row = row0 + r, col = word0 * 4 + c;
+    if (row < rows && col < words_per_row * 4) out_t[col * rows + row] = tile[c][r];
+  }
+}
+
+template <int WORDS, int UNROLL, bool NT>
+void launch_fast(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
+                 int64_t n_words16, int64_t n_ids, hipStream_t stream) {
+  const int64_t n_items = n_words16 / (2 * WORDS);
+  const uint32_t ipg = (uint32_t)(n_ids / (2 * WORDS));
+  int shift = -1;
+  if ((ipg & (ipg - 1)) == 0) shift = __builtin_ctz(ipg);
+  const int64_t per_block = (int64_t)kThreads * UNROLL;
+  const int64_t blocks = (n_items + per_block - 1) / per_block;
+  decompress_kernel<WORDS, UNROLL, NT><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+      reinterpret_cast<const uint32_t *>(packed), reinterpret_cast<const half_t *>(scale),
+      reinterpret_cast<const half_t *>(bias), reinterpret_cast<uint4_t *>(out), n_items, shift, ipg);
+}
+
+}  // namespace
+
+int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
+                      int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed, hipStream_t stream) {
+  const int64_t n_words = rows * n_groups * n_ids;
+  if (n_words == 0) return GQ_OK;
+  if (transposed) {
+    const int64_t words_per_row = n_groups * n_ids;
+    const int64_t gx = (words_per_row + kTileWords - 1) / kTileWords, gy = (rows + kTileRows - 1) / kTileRows;
+    if (gy > 65535) return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: rows=%lld exceeds 65535*64", (long long)rows);
+    decompress_transposed_kernel<<<dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), 0, stream>>>(
+        packed, reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
+        reinterpret_cast<half_t *>(out), rows, words_per_row, n_ids);
+    return check_launch("decompress_transposed_kernel");
+  }
+  const uintptr_t pa = (uintptr_t)packed, oa = (uintptr_t)out;
+  const bool out16 = (oa % 16) == 0;
+  const int variant = option_decompress_variant();
+  // words (32-bit) per work item: the widest of 4/2/1 that divides the group and is aligned
+  int words = 0;
+  if (out16 && n_ids % 8 == 0 && pa % 16 == 0) words = 4;
+  else if (out16 && n_ids % 4 == 0 && pa % 8 == 0) words = 2;
+  else if (out16 && n_ids % 2 == 0 && pa % 4 == 0) words = 1;
+  if (variant >= 100 && variant < 200 && words >= 1) words = 1;       // diagnostic: force 4-byte items
+  if (variant >= 200 && variant < 300 && words >= 2) words = 2;       // diagnostic: force 8-byte items
+  const int sub = variant % 100;
+  if ((n_words + 1) / 2 / kThreads >= (int64_t)1 << 31) return fail(GQ_ERR_UNSUPPORTED, "decompress: tensor too large");
+  if (words == 0) {
+    const int64_t blocks = (n_words + kThreads - 1) / kThreads;
+    decompress_scalar_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+        packed, reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
+        reinterpret_cast<half_t *>(out), n_words, n_ids);
+    return check_launch("decompress_scalar_kernel");
+  }
+#define GQ_DISPATCH(W)                                                                          \
+  switch (sub) {                                                                                \
+    case 1: launch_fast<W, 1, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
+    case 2: launch_fast<W, 2, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
+    case 3: launch_fast<W, 4, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
+    case 4: launch_fast<W, 1, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
+    case 5: launch_fast<W, 2, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
+    case 6: launch_fast<W, 4, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
+    default: launch_fast<W, 2, true>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
+  }
+  if (words == 4) { GQ_DISPATCH(4) }
+  else if (words == 2) { GQ_DISPATCH(2) }
+  else { GQ_DISPATCH(1) }
+#undef GQ_DISPATCH
+  return check_launch("decompress_kernel");
+}
+
+}  // namespace gq

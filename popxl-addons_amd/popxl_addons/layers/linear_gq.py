@@ -1,0 +1,174 @@
+"""Group-quantised linear layer on the GPU (eager), with the constructor, variable names and
+shapes, matmul orientation and `torch_mapping` of the reference's
+popxl_addons/layers/linear_gq.py:19-136."""
+from typing import Optional
+
+import numpy as np
+
+from popxl_addons import _gq_hip
+from popxl_addons.ops.group_quantize_decompress import (
+    group_quantize_compress_numpy,
+    group_quantize_decompress,
+)
+from popxl_addons.utils import NamedTensors, Variable, WeightsDict, _numpy_dtype_of
+
+
+class GroupSizeError(ValueError, ZeroDivisionError):
+    """group_size was left at 0 (the constructor default); the reference fails with a
+    ZeroDivisionError at build time in that case (linear_gq.py:73)."""
+
+
+class LinearGQ:
+    def __init__(
+        self,
+        out_features: int,
+        bias: bool = True,
+        replica_grouping=None,
+        group_size: int = 0,
+        dim: int = -1,
+    ):
+        """
+        Group Quantised Linear layer.
+
+        Stores quantised weights as three variables:
+            weight_compressed: packed integer ids, four 4-bit integers per uint16 element
+            weight_decompression_scale: float16 scale per group
+            weight_decompression_bias: float16 bias per group
+        and an optional additive `bias`.  Variables are zero-initialised on the first build;
+        overwrite them with `load_weights` (see `torch_mapping`).
+
+        Arguments:
+        - out_features (int): output dimension of layer
+        - bias (bool): add a bias term (default True)
+        - replica_grouping: must be None (single GPU, no variable sharding)
+        - group_size (int): values per (scale, bias) pair; must be set to a positive multiple of 4
+        - dim (int): dimension of the [in, out] weight matrix that is grouped.
+                     0: groups run along the input features (fused dequant-matmul kernels);
+                     1 or -1: groups run along the output features.
+        """
+        if replica_grouping is not None:
+            raise NotImplementedError("LinearGQ here runs on one GPU: replica_grouping must be None")
+        self.out_features = out_features
+        self.bias = bias
+        self.replica_grouping = replica_grouping
+        self.group_size = group_size
+        self.dim = dim
+        self.variables: Optional[NamedTensors] = None
+
+    # ----------------------------------------------------------------------------- variables
+
+    def _variable_shapes(self, in_features):
+        # linear_gq.py:59-97
+        if self.group_size == 0:
+            raise GroupSizeError("LinearGQ: group_size is 0; set it to a positive multiple of 4")
+        if self.dim in [1, -1]:
+            compressed_dim, uncompressed_dim = self.out_features, in_features
+        elif self.dim == 0:
+            uncompressed_dim, compressed_dim = self.out_features, in_features
+        else:
+            raise ValueError(f"LinearGQ: dim must be 0, 1 or -1, got {self.dim}")
+        n_groups = compressed_dim // self.group_size
+        return (uncompressed_dim, n_groups, self.group_size // 4), (uncompressed_dim, n_groups, 1)
+
+    def init_variables(self, in_features, dtype, device):
+        import torch
+
+        packed_shape, stat_shape = self._variable_shapes(in_features)
+        named = NamedTensors(
+            weight_compressed=Variable("weight_compressed", torch.zeros(packed_shape, dtype=torch.uint16, device=device)),
+            weight_decompression_scale=Variable(
+                "weight_decompression_scale", torch.zeros(stat_shape, dtype=dtype, device=device)
+            ),
+            weight_decompression_bias=Variable(
+                "weight_decompression_bias", torch.zeros(stat_shape, dtype=dtype, device=device)
+            ),
+        )
+        if self.bias:
+            named.insert("bias", Variable("bias", torch.zeros((self.out_features,), dtype=dtype, device=device)))
+        self.variables = named
+        return named
+
+    def load_weights(self, weights):
+        """Copy a WeightsDict (or a callable producing one from the variables) into the variables."""
+        import torch
+
+        if callable(weights):
+            weights = weights(self.variables)
+        for var, value in weights.items():
+            var.data.copy_(torch.from_numpy(np.ascontiguousarray(value)).to(var.data.device))
+
+    # --------------------------------------------------------------------------------- build
+
+    def build(self, x):
+        """y = x @ decompress(weight) (+ bias), linear_gq.py:99-109.  x: float16 [..., in] on the GPU."""
+        import torch
+
+        if not x.is_cuda:
+            raise RuntimeError("LinearGQ runs on the GPU only: move x to a HIP device")
+        in_features = x.shape[-1]
+        if self.variables is None:
+            self.init_variables(in_features, x.dtype, x.device)
+        v = self.variables
+        if x.dtype != torch.float16 or v.weight_decompression_scale.dtype != torch.float16:
+            raise TypeError("LinearGQ: only float16 activations and float16 scale/bias are supported")
+        packed_shape, _ = self._variable_shapes(in_features)
+        if v.weight_compressed.shape != packed_shape:
+            raise ValueError(f"LinearGQ: x has {in_features} features but weight_compressed is {v.weight_compressed.shape}")
+        b = v.bias.data if self.bias else None
+
+        if self.dim == 0:
+            x2 = x.reshape(-1, in_features).contiguous()
+            with torch.cuda.device(x.device):
+                y = torch.empty((x2.shape[0], self.out_features), dtype=torch.float16, device=x.device)
+                _gq_hip.call(
+                    "gq_linear_f16",
+                    x2.data_ptr(),
+                    x2.shape[0],
+                    v.weight_compressed.data.data_ptr(),
+                    v.weight_decompression_scale.data.data_ptr(),
+                    v.weight_decompression_bias.data.data_ptr(),
+                    0 if b is None else b.data_ptr(),
+                    y.data_ptr(),
+                    self.out_features,
+                    in_features,
+                    self.group_size,
+                    torch.cuda.current_stream(x.device).cuda_stream,
+                )
+            return y.reshape(*x.shape[:-1], self.out_features)
+
+        # groups along the output features: the weight comes out of the decompress kernel as
+        # [in, out] and feeds a dense matmul
+        w = group_quantize_decompress(
+            v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data, self.dim
+        )
+        y = x @ w
+        if b is not None:
+            y = y + b
+        return y
+
+    __call__ = build
+
+    # ------------------------------------------------------------------------- weight mapping
+
+    @staticmethod
+    def torch_mapping(variables: NamedTensors, nn_layer, dtype=None, group_size: int = 64, dim: int = -1) -> WeightsDict:
+        """
+        Mapping from the layer variables to the (compressed) torch.nn.Linear parameters
+        (linear_gq.py:112-136).  `dtype` is the torch dtype of the additive bias (float32 if None).
+        """
+        import torch
+
+        dtype = torch.float32 if dtype is None else dtype
+        state_dict = dict(
+            zip(
+                (
+                    variables.weight_compressed,
+                    variables.weight_decompression_scale,
+                    variables.weight_decompression_bias,
+                ),
+                group_quantize_compress_numpy(nn_layer.weight.T.detach().cpu().numpy(), group_size, dim=dim),
+            )
+        )
+        if "bias" in variables.keys():
+            state_dict[variables.bias] = nn_layer.bias.data.detach().cpu().numpy().astype(_numpy_dtype_of(dtype))
+        return WeightsDict(state_dict)

@@ -1,0 +1,138 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports what the header
+declares, the op wrapper and the layer validate their arguments like the reference."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT
+from popxl_addons import _gq_hip
+from popxl_addons.layers.linear_gq import LinearGQ
+from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy, group_quantize_decompress
+from popxl_addons.utils import NamedTensors, Variable, WeightsDict
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "gq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert len(names) >= 9
+    assert sorted(names) == sorted(_gq_hip.EXPORTS)
+    lib = ctypes.CDLL(_gq_hip.library_path())
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_abi_version_and_error_text_without_gpu():
+    lib = _gq_hip.load()
+    assert lib.gq_abi_version() == _gq_hip.GQ_ABI_VERSION
+    # argument errors are detected before any device call
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_decompress_f16", 0, 0, 0, 0, 4, 4, 4, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER and "NULL" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_decompress_f16", 16, 16, 16, 16, -1, 4, 4, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_decompress_f16", 17, 16, 16, 16, 1, 4, 4, None)
+    assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_f16", 16, 1, 16, 16, 16, 0, 16, 8, 96, 64, None)  # 96 % 64 != 0
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_f16", 16, 17, 16, 16, 16, 0, 16, 8, 64, 64, None)  # m_rows > 16
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_f16", 16, 1, 16, 16, 16, 0, 16, 8, 64, 6, None)  # group_size % 4
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_set_option", b"no_such_option", 1)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED
+    # zero-sized problems succeed without touching a device
+    _gq_hip.call("gq_decompress_f16", 0, 0, 0, 0, 0, 4, 4, None)
+    _gq_hip.call("gq_gemv_f16", 0, 0, 0, 0, 0, 0, 0, 8, 64, 64, None)
+    _gq_hip.call("gq_compress_f16", 0, 0, 0, 0, 0, 0, 4, 64, None)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setenv("GQ_HIP_LIBRARY", "/nonexistent/libgq_hip.so")
+    monkeypatch.setattr(_gq_hip, "_lib", None)
+    with pytest.raises(ImportError):
+        _gq_hip.load()
+
+
+def test_op_argument_validation():
+    """Exceptions of the reference wrapper (group_quantize_decompress.py:57-73) and of
+    GroupQuantizeDecompressOp::setup (group_quantize_decompress.cpp:41-63)."""
+    t = torch.zeros((4, 2, 3), dtype=torch.uint16)
+    s = torch.zeros((4, 2, 1), dtype=torch.float16)
+    with pytest.raises(NotImplementedError):
+        group_quantize_decompress(torch.zeros((4, 6), dtype=torch.uint16), s, s)
+    with pytest.raises(NotImplementedError):
+        group_quantize_decompress(torch.zeros((1, 4, 2, 3), dtype=torch.uint16), s, s)
+    with pytest.raises(ValueError, match="group_scale.rank"):
+        group_quantize_decompress(t, torch.zeros((4,), dtype=torch.float16), s)
+    with pytest.raises(ValueError, match="group_bias.rank"):
+        group_quantize_decompress(t, s, torch.zeros((4, 2, 1, 1), dtype=torch.float16))
+    with pytest.raises(ValueError, match="t and group_scale"):
+        group_quantize_decompress(t, torch.zeros((4, 3, 1), dtype=torch.float16), s)
+    with pytest.raises(ValueError, match="t and group_bias"):
+        group_quantize_decompress(t, s, torch.zeros((5, 2), dtype=torch.float16))
+    with pytest.raises(ValueError, match="last dimension"):
+        group_quantize_decompress(t, torch.zeros((4, 2, 2), dtype=torch.float16), s)
+    # rank-2 scale/bias are accepted (reshaped to (..., 1)); a CPU tensor is then refused: no fallback
+    with pytest.raises(RuntimeError, match="GPU only"):
+        group_quantize_decompress(t, torch.zeros((4, 2), dtype=torch.float16), s)
+
+
+def test_linear_gq_variables_and_mapping():
+    """Variable names, shapes and dtypes of LinearGQ.build (linear_gq.py:67-108) and torch_mapping (:112-136)."""
+    torch.manual_seed(0)
+    nn_layer = torch.nn.Linear(128, 256, bias=True)
+    for dim, packed_shape in ((0, (256, 8, 4)), (-1, (128, 16, 4)), (1, (128, 16, 4))):
+        layer = LinearGQ(256, bias=True, group_size=16, dim=dim)
+        v = layer.init_variables(128, torch.float16, "cpu")
+        assert list(v.keys()) == ["weight_compressed", "weight_decompression_scale", "weight_decompression_bias", "bias"]
+        assert v.weight_compressed.shape == packed_shape and v.weight_compressed.dtype == torch.uint16
+        assert v.weight_decompression_scale.shape == (*packed_shape[:2], 1)
+        assert v.weight_decompression_bias.dtype == torch.float16 and v.bias.shape == (256,)
+        w = LinearGQ.torch_mapping(v, nn_layer, dtype=torch.float16, group_size=16, dim=dim)
+        assert len(w) == 4
+        want = group_quantize_compress_numpy(nn_layer.weight.T.detach().numpy(), 16, dim=dim)
+        assert np.array_equal(w[v.weight_compressed], want[0])
+        layer.load_weights(w)
+        assert np.array_equal(v.weight_compressed.data.numpy(), want[0])
+    assert "bias" not in LinearGQ(8, bias=False, group_size=4).init_variables(8, torch.float16, "cpu")
+
+
+def test_linear_gq_misuse():
+    with pytest.raises(ZeroDivisionError):  # group_size left at its default 0 (linear_gq.py:25,73)
+        LinearGQ(8).init_variables(8, torch.float16, "cpu")
+    with pytest.raises(NotImplementedError):
+        LinearGQ(8, replica_grouping=object(), group_size=4)
+    with pytest.raises(ValueError):
+        LinearGQ(8, group_size=4, dim=2).init_variables(8, torch.float16, "cpu")
+    with pytest.raises(RuntimeError, match="GPU only"):
+        LinearGQ(8, group_size=4, dim=0).build(torch.zeros((1, 8), dtype=torch.float16))
+
+
+def test_weights_dict_validates_dtype_and_shape():
+    """popxl_addons/utils.py:91-99."""
+    var = Variable("w", torch.zeros((2, 3), dtype=torch.float16))
+    d = WeightsDict()
+    d[var] = np.zeros((2, 3), np.float16)
+    with pytest.raises(ValueError, match="dtypes"):
+        d[var] = np.zeros((2, 3), np.float32)
+    with pytest.raises(ValueError, match="shapes"):
+        d[var] = np.zeros((3, 2), np.float16)
+    nt = NamedTensors(w=var)
+    assert nt.w is var and nt["w"] is var and "w" in nt
+    with pytest.raises(AttributeError):
+        nt.missing
