@@ -103,7 +103,7 @@ def group_quantize_decompress(t, group_scale, group_bias, dim=-1):
     rows, n_groups, n_ids = t.shape
     n_cols = n_groups * n_ids * 4
 
-    transposed = _perm_last_to(2, dim) != [0, 1]
+    transposed = dim != -1 and _perm_last_to(2, dim) != [0, 1]
     with torch.cuda.device(t.device):
         out = torch.empty((n_cols, rows) if transposed else (rows, n_cols), dtype=torch.float16, device=t.device)
         _gq_hip.call(
