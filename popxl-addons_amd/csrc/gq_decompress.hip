@@ -60,37 +60,39 @@ __device__ __forceinline__ T load_packed(const T *p) {
 // (WORDS in {1, 2, 4}: a 4/8/16-byte load) -> WORDS 16-byte stores.  All words of an item
 // lie in one group (the launcher guarantees WORDS divides the words per group), so an item
 // needs one (scale, bias) pair.  Items are dealt to lanes so that consecutive lanes take
-// consecutive items: loads and stores of a wave are contiguous.
-template <int WORDS, int UNROLL, bool NT>
-__global__ __launch_bounds__(kThreads) void decompress_kernel(const uint32_t *__restrict__ packed,
-                                                              const half_t *__restrict__ scale,
-                                                              const half_t *__restrict__ bias,
-                                                              uint4_t *__restrict__ out, int64_t n_items,
-                                                              int items_per_group_shift,
-                                                              uint32_t items_per_group) {
+// consecutive items: with WORDS == 1 every load and store instruction of a wave covers one
+// contiguous span (256 B read, 1 KiB written).  A workgroup walks the tensor with a grid
+// stride of THREADS * UNROLL items; the launcher picks the grid (one pass or persistent).
+template <int THREADS, int WORDS, int UNROLL, bool NT_LOAD, bool NT_STORE>
+__global__ __launch_bounds__(THREADS) void decompress_kernel(const uint32_t *__restrict__ packed,
+                                                             const half_t *__restrict__ scale,
+                                                             const half_t *__restrict__ bias,
+                                                             uint4_t *__restrict__ out, int64_t n_items,
+                                                             int items_per_group_shift) {
   typedef uint32_t vec_t __attribute__((ext_vector_type(WORDS)));
-  const int64_t base = (int64_t)blockIdx.x * (kThreads * UNROLL) + threadIdx.x;
-  vec_t w[UNROLL];
-  half_t s[UNROLL], b[UNROLL];
+  const int64_t stride = (int64_t)gridDim.x * (THREADS * UNROLL);
+  for (int64_t base = (int64_t)blockIdx.x * (THREADS * UNROLL) + threadIdx.x; base < n_items; base += stride) {
+    vec_t w[UNROLL];
+    half_t s[UNROLL], b[UNROLL];
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    const int64_t item = base + (int64_t)u * kThreads;
-    if (item < n_items) {
-      w[u] = load_packed<vec_t, NT>(reinterpret_cast<const vec_t *>(packed) + item);
-      const int64_t group =
-          items_per_group_shift >= 0 ? (item >> items_per_group_shift) : (item / items_per_group);
-      s[u] = scale[group];
-      b[u] = bias[group];
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t item = base + (int64_t)u * THREADS;
+      if (item < n_items) {
+        w[u] = load_packed<vec_t, NT_LOAD>(reinterpret_cast<const vec_t *>(packed) + item);
+        const int64_t group = item >> items_per_group_shift;
+        s[u] = scale[group];
+        b[u] = bias[group];
+      }
     }
-  }
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    const int64_t item = base + (int64_t)u * kThreads;
-    if (item < n_items) {
-      const half2_t s2 = {s[u], s[u]}, b2 = {b[u], b[u]};
-      uint4_t *dst = out + item * WORDS;
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t item = base + (int64_t)u * THREADS;
+      if (item < n_items) {
+        const half2_t s2 = {s[u], s[u]}, b2 = {b[u], b[u]};
+        uint4_t *dst = out + item * WORDS;
 #pragma unroll
-      for (int k = 0; k < WORDS; ++k) store16<NT>(dst + k, expand_word(w[u][k], s2, b2));
+        for (int k = 0; k < WORDS; ++k) store16<NT_STORE>(dst + k, expand_word(w[u][k], s2, b2));
+      }
     }
   }
 }
@@ -146,18 +148,16 @@ __global__ __launch_bounds__(kThreads) void decompress_transposed_kernel(
   }
 }
 
-template <int WORDS, int UNROLL, bool NT>
+template <int THREADS, int WORDS, int UNROLL, bool NT_LOAD, bool NT_STORE>
 void launch_fast(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
-                 int64_t n_words16, int64_t n_ids, hipStream_t stream) {
+                 int64_t n_words16, int shift, int64_t max_blocks, hipStream_t stream) {
   const int64_t n_items = n_words16 / (2 * WORDS);
-  const uint32_t ipg = (uint32_t)(n_ids / (2 * WORDS));
-  int shift = -1;
-  if ((ipg & (ipg - 1)) == 0) shift = __builtin_ctz(ipg);
-  const int64_t per_block = (int64_t)kThreads * UNROLL;
-  const int64_t blocks = (n_items + per_block - 1) / per_block;
-  decompress_kernel<WORDS, UNROLL, NT><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+  const int64_t per_block = (int64_t)THREADS * UNROLL;
+  int64_t blocks = (n_items + per_block - 1) / per_block;
+  if (max_blocks > 0 && blocks > max_blocks) blocks = max_blocks;
+  decompress_kernel<THREADS, WORDS, UNROLL, NT_LOAD, NT_STORE><<<dim3((unsigned)blocks), dim3(THREADS), 0, stream>>>(
       reinterpret_cast<const uint32_t *>(packed), reinterpret_cast<const half_t *>(scale),
-      reinterpret_cast<const half_t *>(bias), reinterpret_cast<uint4_t *>(out), n_items, shift, ipg);
+      reinterpret_cast<const half_t *>(bias), reinterpret_cast<uint4_t *>(out), n_items, shift);
 }
 
 }  // namespace
@@ -178,14 +178,16 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
   const uintptr_t pa = (uintptr_t)packed, oa = (uintptr_t)out;
   const bool out16 = (oa % 16) == 0;
   const int variant = option_decompress_variant();
-  // words (32-bit) per work item: the widest of 4/2/1 that divides the group and is aligned
-  int words = 0;
-  if (out16 && n_ids % 8 == 0 && pa % 16 == 0) words = 4;
-  else if (out16 && n_ids % 4 == 0 && pa % 8 == 0) words = 2;
-  else if (out16 && n_ids % 2 == 0 && pa % 4 == 0) words = 1;
-  if (variant >= 100 && variant < 200 && words >= 1) words = 1;       // diagnostic: force 4-byte items
-  if (variant >= 200 && variant < 300 && words >= 2) words = 2;       // diagnostic: force 8-byte items
-  const int sub = variant % 100;
+  // 32-bit words per work item: 1 unless a diagnostic variant asks for wider items.  Items must
+  // tile a group (power-of-two count per group so the group index is a shift) and be aligned.
+  auto usable = [&](int words) {
+    if (!out16 || n_ids % (2 * words) != 0 || pa % (4 * words) != 0) return false;
+    const int64_t ipg = n_ids / (2 * words);
+    return (ipg & (ipg - 1)) == 0;
+  };
+  int words = usable(1) ? 1 : 0;
+  if (variant >= 200 && variant < 300 && usable(2)) words = 2;
+  if (variant >= 400 && variant < 500 && usable(4)) words = 4;
   if ((n_words + 1) / 2 / kThreads >= (int64_t)1 << 31) return fail(GQ_ERR_UNSUPPORTED, "decompress: tensor too large");
   if (words == 0) {
     const int64_t blocks = (n_words + kThreads - 1) / kThreads;
@@ -194,20 +196,39 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
         reinterpret_cast<half_t *>(out), n_words, n_ids);
     return check_launch("decompress_scalar_kernel");
   }
-#define GQ_DISPATCH(W)                                                                          \
-  switch (sub) {                                                                                \
-    case 1: launch_fast<W, 1, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
-    case 2: launch_fast<W, 2, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
-    case 3: launch_fast<W, 4, false>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
-    case 4: launch_fast<W, 1, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
-    case 5: launch_fast<W, 2, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
-    case 6: launch_fast<W, 4, true>(packed, scale, bias, out, n_words, n_ids, stream); break;   \
-    default: launch_fast<W, 2, true>(packed, scale, bias, out, n_words, n_ids, stream); break;  \
+  const int shift = __builtin_ctzll((unsigned long long)(n_ids / (2 * words)));
+  const int sub = variant % 100;
+#define GQ_ARGS packed, scale, bias, out, n_words, shift
+  if (words == 4) {
+    launch_fast<256, 4, 1, false, false>(GQ_ARGS, 0, stream);
+  } else if (words == 2) {
+    launch_fast<256, 2, 1, false, true>(GQ_ARGS, 0, stream);
+  } else {
+    switch (sub) {
+      case 1: launch_fast<256, 1, 1, false, false>(GQ_ARGS, 0, stream); break;
+      case 2: launch_fast<256, 1, 1, true, false>(GQ_ARGS, 0, stream); break;
+      case 3: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+      case 4: launch_fast<256, 1, 1, true, true>(GQ_ARGS, 0, stream); break;
+      case 5: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+      case 6: launch_fast<1024, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+      case 7: launch_fast<128, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+      case 8: launch_fast<64, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+      case 9: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
+      case 10: launch_fast<256, 1, 4, false, true>(GQ_ARGS, 0, stream); break;
+      case 11: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 8, stream); break;
+      case 12: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 16, stream); break;
+      case 13: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 32, stream); break;
+      case 14: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 256 * 4, stream); break;
+      case 15: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 256 * 8, stream); break;
+      case 16: launch_fast<1024, 1, 1, false, true>(GQ_ARGS, 256 * 2, stream); break;
+      case 17: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 256 * 8, stream); break;
+      case 18: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 256 * 16, stream); break;
+      case 19: launch_fast<512, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
+      case 20: launch_fast<128, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
+      default: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
+    }
   }
-  if (words == 4) { GQ_DISPATCH(4) }
-  else if (words == 2) { GQ_DISPATCH(2) }
-  else { GQ_DISPATCH(1) }
-#undef GQ_DISPATCH
+#undef GQ_ARGS
   return check_launch("decompress_kernel");
 }
 

@@ -23,26 +23,34 @@ __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_c
 // a workgroup take interleaved chunks of the same 16 rows and their partial sums meet in LDS.
 // ---------------------------------------------------------------------------------------
 
+// (w & mask) | magic in one VALU op; mask and magic live in VGPRs (one constant-bus operand is
+// all a VOP3 instruction may take on this target).
+__device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "v"(mask), "v"(magic));
+  return r;
+}
+
 // 8 codes of `w` -> 8 fp16 weights, order (0,4,1,5,2,6,3,7).  The nibble is or-ed into the
 // mantissa of 1024.0 (ulp 1) or, for nibbles sitting at bits 7:4, read as 1024 + 16*code; both
-// are brought back to the exact code with one packed op, then scaled with a packed fma.
+// are brought back to the exact code with one packed op, then scaled with a packed fma:
+// 13 VALU instructions per 8 weights.
 __device__ __forceinline__ half8_t dequant_word(uint32_t w, half2_t s2, half2_t b2) {
   const half2_t kNeg1024 = {(half_t)-1024.0f, (half_t)-1024.0f};
   const half2_t kSixteenth = {(half_t)0.0625f, (half_t)0.0625f};
   const half2_t kNeg64 = {(half_t)-64.0f, (half_t)-64.0f};
+  const uint32_t kLo = 0x000F000Fu, kHi = 0x00F000F0u, kMagic = 0x64006400u;
   const uint32_t hi = w >> 8;
-  const half2_t c0 = __builtin_elementwise_fma(as_half2((hi & 0x00F000F0u) | 0x64006400u), kSixteenth, kNeg64);
-  const half2_t c1 = as_half2((hi & 0x000F000Fu) | 0x64006400u) + kNeg1024;
-  const half2_t c2 = __builtin_elementwise_fma(as_half2((w & 0x00F000F0u) | 0x64006400u), kSixteenth, kNeg64);
-  const half2_t c3 = as_half2((w & 0x000F000Fu) | 0x64006400u) + kNeg1024;
+  const half2_t c0 = __builtin_elementwise_fma(as_half2(and_or(hi, kHi, kMagic)), kSixteenth, kNeg64);
+  const half2_t c1 = as_half2(and_or(hi, kLo, kMagic)) + kNeg1024;
+  const half2_t c2 = __builtin_elementwise_fma(as_half2(and_or(w, kHi, kMagic)), kSixteenth, kNeg64);
+  const half2_t c3 = as_half2(and_or(w, kLo, kMagic)) + kNeg1024;
   const half2_t w0 = __builtin_elementwise_fma(c0, s2, b2);
   const half2_t w1 = __builtin_elementwise_fma(c1, s2, b2);
   const half2_t w2 = __builtin_elementwise_fma(c2, s2, b2);
   const half2_t w3 = __builtin_elementwise_fma(c3, s2, b2);
-  half8_t r;
-  r[0] = w0[0]; r[1] = w0[1]; r[2] = w1[0]; r[3] = w1[1];
-  r[4] = w2[0]; r[5] = w2[1]; r[6] = w3[0]; r[7] = w3[1];
-  return r;
+  return __builtin_shufflevector(__builtin_shufflevector(w0, w1, 0, 1, 2, 3),
+                                 __builtin_shufflevector(w2, w3, 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // 8 consecutive fp16 of x -> order (0,4,1,5,2,6,3,7)
@@ -55,71 +63,130 @@ __device__ __forceinline__ half8_t permute_x(uint4_t q) {
   return __builtin_bit_cast(half8_t, p);
 }
 
-template <int NWAVES>
+// One chunk = 512 contraction indices = four 16-byte loads per lane and row block ("slots" of
+// 128 indices: lane (r, kc) takes bytes [64 * slot + 16 * kc, +16) of its row's chunk).
+// R     row blocks of 16 rows handled by one wave with the same x fragments (x is loaded and
+//       permuted once per chunk, then reused R times).
+// GS    64 or 128: scale/bias of a chunk are fetched as one 16/8-byte load per row and the lane's
+//       value is picked with a byte permute; 0: any power-of-two group >= 32, 2-byte loads.
+// FULL  k_in is a multiple of 512 (no slot predication).
+template <int NWAVES, int R, int GS, bool FULL>
 __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
     int gs_shift) {
-  __shared__ float4_t partial[NWAVES][64];
+  __shared__ float4_t partial[NWAVES][R][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kc = lane >> 4;
-  const int row = min((int)blockIdx.x * 16 + r, n_out - 1);
-  const int n_slots = k_in >> 7;  // 128 contraction indices = 4 lanes x 16 bytes per row
+  const int n_slots = k_in >> 7;
+  const int n_chunks = (n_slots + 3) >> 2;
   const int groups_per_row = k_in >> gs_shift;
-  const uint4_t *wrow = packed + (int64_t)row * (k_in >> 5);
-  const half_t *srow = scale + (int64_t)row * groups_per_row;
-  const half_t *brow = bias + (int64_t)row * groups_per_row;
   const bool has_x = r < m_rows;
-  const half_t *xrow = x + (int64_t)(has_x ? r : 0) * k_in;
+  const half_t *xrow = x + (int64_t)(has_x ? r : 0) * k_in + kc * 32;
+  const uint4_t *wrow[R];
+  const half_t *srow[R], *brow[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int row = min(((int)blockIdx.x * R + i) * 16 + r, n_out - 1);
+    wrow[i] = packed + (int64_t)row * (k_in >> 5) + kc;
+    srow[i] = scale + (int64_t)row * groups_per_row;
+    brow[i] = bias + (int64_t)row * groups_per_row;
+  }
+  // byte selector that broadcasts the low or the high half of a 32-bit word (GS == 64: the lane's
+  // group within a slot is kc / 2)
+  const uint32_t half_sel = (kc & 2) ? 0x07060706u : 0x05040504u;
 
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
-  for (int c = wave; c * 4 < n_slots; c += NWAVES) {
-    uint4_t wq[4], xq[4][4];
-    half_t sc[4], bi[4];
+  float4_t acc[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int c = wave; c < n_chunks; c += NWAVES) {
+    uint4_t wq[R][4];
+    uint32_t s2[R][4], b2[R][4];  // (scale, scale) and (bias, bias) as packed fp16 pairs
+    // ---- issue every load of the chunk
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int slot = c * 4 + j;
+        if (FULL || slot < n_slots)
+          wq[i][j] = __builtin_nontemporal_load(wrow[i] + slot * 4);
+        else
+          wq[i][j] = uint4_t{0u, 0u, 0u, 0u};
+      }
+      if constexpr (GS == 64) {
+        const uint4_t sv = *reinterpret_cast<const uint4_t *>(srow[i] + c * 8);
+        const uint4_t bv = *reinterpret_cast<const uint4_t *>(brow[i] + c * 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          s2[i][j] = __builtin_amdgcn_perm(sv[j], sv[j], half_sel);
+          b2[i][j] = __builtin_amdgcn_perm(bv[j], bv[j], half_sel);
+        }
+      } else if constexpr (GS == 128) {
+        const uint2_t sv = *reinterpret_cast<const uint2_t *>(srow[i] + c * 4);
+        const uint2_t bv = *reinterpret_cast<const uint2_t *>(brow[i] + c * 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t sel = (j & 1) ? 0x07060706u : 0x05040504u;
+          s2[i][j] = __builtin_amdgcn_perm(sv[j >> 1], sv[j >> 1], sel);
+          b2[i][j] = __builtin_amdgcn_perm(bv[j >> 1], bv[j >> 1], sel);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int slot = c * 4 + j;
+          uint32_t sv = 0, bv = 0;
+          if (FULL || slot < n_slots) {
+            const int g = (slot * 128 + kc * 32) >> gs_shift;
+            sv = __builtin_bit_cast(uint16_t, srow[i][g]);
+            bv = __builtin_bit_cast(uint16_t, brow[i][g]);
+          }
+          s2[i][j] = sv | (sv << 16);
+          b2[i][j] = bv | (bv << 16);
+        }
+      }
+    }
+    half8_t xp[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int slot = c * 4 + j;
-      const bool valid = slot < n_slots;
-      const int k0 = slot * 128 + kc * 32;
-      wq[j] = uint4_t{0u, 0u, 0u, 0u};
-      sc[j] = (half_t)0.f;
-      bi[j] = (half_t)0.f;
-      if (valid) {
-        wq[j] = __builtin_nontemporal_load(wrow + slot * 4 + kc);
-        sc[j] = srow[k0 >> gs_shift];
-        bi[j] = brow[k0 >> gs_shift];
-      }
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        xq[j][s] = uint4_t{0u, 0u, 0u, 0u};
-        if (valid && has_x) xq[j][s] = *reinterpret_cast<const uint4_t *>(xrow + k0 + s * 8);
+        uint4_t q = {0u, 0u, 0u, 0u};
+        if (has_x && (FULL || slot < n_slots)) q = *reinterpret_cast<const uint4_t *>(xrow + slot * 128 + s * 8);
+        xp[j][s] = permute_x(q);
       }
     }
+    // ---- expand and multiply
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const half2_t s2 = {sc[j], sc[j]}, b2 = {bi[j], bi[j]};
+    for (int i = 0; i < R; ++i)
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const half8_t a = dequant_word(wq[j][s], s2, b2);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, permute_x(xq[j][s]), acc, 0, 0, 0);
-      }
-    }
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const half8_t a = dequant_word(wq[i][j][s], as_half2(s2[i][j]), as_half2(b2[i][j]));
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xp[j][s], acc[i], 0, 0, 0);
+        }
   }
-  partial[wave][lane] = acc;
+#pragma unroll
+  for (int i = 0; i < R; ++i) partial[wave][i][lane] = acc[i];
   __syncthreads();
-  if (wave == 0) {
-    float4_t sum = partial[0][lane];
+  // lane holds D[n = 4 * kc + e][m = r] of row block i
+  for (int t = threadIdx.x; t < R * 64; t += NWAVES * 64) {
+    const int i = t >> 6, l = t & 63;
+    float4_t sum = partial[0][i][l];
 #pragma unroll
-    for (int w = 1; w < NWAVES; ++w) sum += partial[w][lane];
-    // lane holds D[n = 4*kc + i][m = r]
-    if (r < m_rows) {
+    for (int w = 1; w < NWAVES; ++w) sum += partial[w][i][l];
+    const int m = l & 15;
+    if (m < m_rows) {
+      const int n0 = ((int)blockIdx.x * R + i) * 16 + 4 * (l >> 4);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = (int)blockIdx.x * 16 + 4 * kc + i;
+      for (int e = 0; e < 4; ++e) {
+        const int n = n0 + e;
         if (n < n_out) {
-          float v = sum[i];
+          float v = sum[e];
           if (out_bias) v += (float)out_bias[n];
-          y[(int64_t)r * n_out + n] = (half_t)v;
+          y[(int64_t)m * n_out + n] = (half_t)v;
         }
       }
     }
@@ -186,11 +253,39 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
                        ((uintptr_t)packed % 16) == 0;
   if (fast_ok && variant != 1) {
     const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
-    const unsigned blocks = (unsigned)((n_out + 15) / 16);
-    gemv_mfma_kernel<8><<<dim3(blocks), dim3(512), 0, stream>>>(
-        reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
-        reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
-        reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift);
+    const int64_t row_blocks = (n_out + 15) / 16;
+    const bool full = k_in % 512 == 0;
+    // rows per wave: reuse the permuted x fragments as often as the row count allows while still
+    // filling 256 compute units
+    int r = row_blocks >= 1024 ? 4 : (row_blocks >= 512 ? 2 : 1);
+    if (variant >= 10 && variant < 20) r = variant == 11 ? 1 : (variant == 12 ? 2 : 4);
+    const int gs_mode = (group_size == 64 && full) ? 64 : ((group_size == 128 && full) ? 128 : 0);
+    const unsigned blocks = (unsigned)((row_blocks + r - 1) / r);
+#define GQ_GEMV_ARGS                                                                                      \
+  reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \
+      reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),                    \
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift
+#define GQ_GEMV_LAUNCH(NW, R, GS, FULL) \
+  gemv_mfma_kernel<NW, R, GS, FULL><<<dim3(blocks), dim3(NW * 64), 0, stream>>>(GQ_GEMV_ARGS)
+#define GQ_GEMV_BY_R(NW, GS, FULL)                      \
+  do {                                                  \
+    if (r == 4) GQ_GEMV_LAUNCH(NW, 4, GS, FULL);        \
+    else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL);   \
+    else GQ_GEMV_LAUNCH(NW, 1, GS, FULL);               \
+  } while (0)
+    if (gs_mode == 64) {
+      if (r == 1 && k_in >= 8192) GQ_GEMV_LAUNCH(16, 1, 64, true);
+      else GQ_GEMV_BY_R(8, 64, true);
+    } else if (gs_mode == 128) {
+      GQ_GEMV_BY_R(8, 128, true);
+    } else if (full) {
+      GQ_GEMV_BY_R(8, 0, true);
+    } else {
+      GQ_GEMV_BY_R(8, 0, false);
+    }
+#undef GQ_GEMV_BY_R
+#undef GQ_GEMV_LAUNCH
+#undef GQ_GEMV_ARGS
     return check_launch("gemv_mfma_kernel");
   }
   const unsigned blocks = (unsigned)((n_out + 3) / 4);
