@@ -138,6 +138,391 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const half_t *__restrict
     }
 }
 
+
+// (w & mask) | magic in one VALU op; mask and magic live in VGPRs.
+__device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "v"(mask), "v"(magic));
+  return r;
+}
+
+// codes (2p, 2p+1) of a word sit in one byte: byte 1, 0, 3, 2 for p = 0..3, high nibble first.
+// The byte is copied to byte 0 and byte 2 of a register; masking 0x000F00F0 leaves code 2p at
+// bits 7:4 of the low half (read as 1024 + 16 c) and code 2p+1 at bits 3:0 of the high half
+// (1024 + c); one packed fma with (1/16, 1) and (-64, -1024) makes both exact.
+__device__ __forceinline__ half8_t dequant_word_natural(uint32_t w, half2_t s2, half2_t b2) {
+  const half2_t kMul = {(half_t)0.0625f, (half_t)1.0f};
+  const half2_t kAdd = {(half_t)-64.0f, (half_t)-1024.0f};
+  const uint32_t kMask = 0x000F00F0u, kMagic = 0x64006400u;
+  const uint32_t t0 = __builtin_amdgcn_perm(0u, w, 0x0c010c01u);
+  const uint32_t t1 = __builtin_amdgcn_perm(0u, w, 0x0c000c00u);
+  const uint32_t t2 = __builtin_amdgcn_perm(0u, w, 0x0c030c03u);
+  const uint32_t t3 = __builtin_amdgcn_perm(0u, w, 0x0c020c02u);
+  const half2_t c0 = __builtin_elementwise_fma(as_half2(and_or(t0, kMask, kMagic)), kMul, kAdd);
+  const half2_t c1 = __builtin_elementwise_fma(as_half2(and_or(t1, kMask, kMagic)), kMul, kAdd);
+  const half2_t c2 = __builtin_elementwise_fma(as_half2(and_or(t2, kMask, kMagic)), kMul, kAdd);
+  const half2_t c3 = __builtin_elementwise_fma(as_half2(and_or(t3, kMask, kMagic)), kMul, kAdd);
+  const half2_t w0 = __builtin_elementwise_fma(c0, s2, b2);
+  const half2_t w1 = __builtin_elementwise_fma(c1, s2, b2);
+  const half2_t w2 = __builtin_elementwise_fma(c2, s2, b2);
+  const half2_t w3 = __builtin_elementwise_fma(c3, s2, b2);
+  return __builtin_shufflevector(__builtin_shufflevector(w0, w1, 0, 1, 2, 3),
+                                 __builtin_shufflevector(w2, w3, 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// s_waitcnt lgkmcnt(n) that also "touches" a register tuple, so that instructions consuming the
+// tuple cannot be scheduled above the wait
+template <int N>
+__device__ __forceinline__ void wait_lds(uint4_t &a) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
+}
+
+// ---------------------------------------------------------------------------------------
+// Pipelined kernel for large batches.
+//
+// Workgroup = WM x WN waves; a wave owns FM x FN accumulators of 32 x 32 (v_mfma_f32_32x32x16_f16),
+// i.e. a (32 FM) x (32 FN) sub-tile; K advances 64 at a time ("tile").
+//
+// Data flow.  Everything that comes from global memory goes straight into LDS with
+// global_load_lds_* (no VGPR staging), two tiles ahead, and is read back with ds_read instructions
+// issued from inline assembly and waited for explicitly.  The compiler therefore never sees a
+// register with a load in flight: its own wait insertion is conservative across the loop back edge
+// and cannot tell ring stages apart, and would drain the whole prefetch queue (vmcnt(0)) once per
+// iteration.
+//   x tile  : XS-stage ring shared by the workgroup.  A row is 8 chunks of 16 bytes; chunk c of row
+//             r sits at chunk slot c ^ ((r >> 1) & 7), so the 16-byte fragment reads of 16
+//             consecutive rows cover all 64 LDS banks once (measured: zero bank conflicts).  The
+//             swizzle is applied by choosing each lane's source address.
+//   weights : 3-stage ring private to each wave.  Lane (n, h) owns the 16 bytes = 32 codes of row n
+//             that start at index 32 h of the tile; lanes with h == 0 also fetch the dword holding
+//             the row's scale and the one holding its bias.  One 32-bit word per MFMA step is
+//             expanded into the B operand in memory order: per pair of codes one byte permute, one
+//             and-or into the mantissa of 1024.0, one packed fma that recovers the exact codes,
+//             one packed fma with (scale, bias) -- 16 VALU instructions per 8 weights.
+//   MFMA step s of a tile contracts indices {32 h + 8 s + i}: lane (m, h) of the A operand reads
+//   chunk 4 h + s of its row.
+//
+// Schedule of a tile (4 MFMA steps):
+//   * steps 0..2 are FM groups of {FN MFMAs, one A-fragment read for the next step, one
+//     direct-to-LDS load of the tile two ahead, a slice of the next step's dequantisation}, fenced
+//     with sched_barrier so the compiler keeps the interleaving.  Loads are never issued as a
+//     burst: eight waves issuing a whole tile at once block each other behind the 64 B/clk
+//     address path of the compute unit for ~1000 cycles.
+//   * before step 3 comes the only workgroup barrier of the tile: every wave has waited for its
+//     own LDS reads of this tile and for its own loads of the next one, so after the barrier the
+//     next tile is readable and this tile's x stage may be overwritten.  The next tile's weights,
+//     first A fragments and first B operand are fetched and built under the MFMAs of step 3.
+// ---------------------------------------------------------------------------------------
+constexpr int kWStages = 3;
+
+template <int WM, int WN, int FM, int FN, int XS>
+struct Pipe2Shape {
+  static constexpr int NW = WM * WN, TM = 32 * FM, TN = 32 * FN, TILE_M = WM * TM, TILE_N = WN * TN;
+  static constexpr int X_STAGE = TILE_M * 128, W_STAGE = FN * 1280;
+  static constexpr int X_BYTES = XS * X_STAGE, LDS_BYTES = X_BYTES + NW * kWStages * W_STAGE;
+  static constexpr int A_OPS = TILE_M / 8 / NW;
+  static constexpr int OPS = A_OPS + 3 * FN;
+};
+
+// The 16 VALU instructions that turn one packed word into a B operand, cut into PIECES slices so
+// that they can be spread between MFMAs.  State: t (permuted bytes / raw halves), c (exact codes).
+struct DequantState {
+  uint32_t t[4];
+  half2_t c[4];
+  half2_t w[4];
+};
+
+template <int PIECES>
+__device__ __forceinline__ void dequant_piece(int piece, uint32_t word, half2_t s2, half2_t z2, DequantState &st) {
+  const half2_t kMul = {(half_t)0.0625f, (half_t)1.0f};
+  const half2_t kAdd = {(half_t)-64.0f, (half_t)-1024.0f};
+  const uint32_t kMask = 0x000F00F0u, kMagic = 0x64006400u;
+  const uint32_t sel[4] = {0x0c010c01u, 0x0c000c00u, 0x0c030c03u, 0x0c020c02u};
+  // operation o of pair p: 0 byte permute, 1 and-or into 1024.0, 2 exact code, 3 scale and bias
+#pragma unroll
+  for (int op = 0; op < 16; ++op) {
+    if (op * PIECES / 16 != piece) continue;
+    const int p = op >> 2, o = op & 3;
+    if (o == 0) st.t[p] = __builtin_amdgcn_perm(0u, word, sel[p]);
+    if (o == 1) st.t[p] = and_or(st.t[p], kMask, kMagic);
+    if (o == 2) st.c[p] = __builtin_elementwise_fma(as_half2(st.t[p]), kMul, kAdd);
+    if (o == 3) st.w[p] = __builtin_elementwise_fma(st.c[p], s2, z2);
+  }
+}
+
+__device__ __forceinline__ half8_t dequant_result(const DequantState &st) {
+  return __builtin_shufflevector(__builtin_shufflevector(st.w[0], st.w[1], 0, 1, 2, 3),
+                                 __builtin_shufflevector(st.w[2], st.w[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <int WM, int WN, int FM, int FN, int XS>
+__device__ __forceinline__ void gemm_pipe2_body(
+    const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
+    const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
+    int gs_shift) {
+  using S = Pipe2Shape<WM, WN, FM, FN, XS>;
+  constexpr int NW = S::NW, TM = S::TM, TN = S::TN, TILE_M = S::TILE_M, TILE_N = S::TILE_N;
+  constexpr int A_OPS = S::A_OPS, OPS = S::OPS;
+  static_assert(TILE_M % (8 * NW) == 0, "x tile must split evenly over the waves");
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int m0 = blockIdx.y * TILE_M, n0 = blockIdx.x * TILE_N;
+  const int groups_per_row = k_in >> gs_shift;
+  const int n_tiles = k_in >> 6;
+
+  const half_t *a_src[A_OPS];
+#pragma unroll
+  for (int q = 0; q < A_OPS; ++q) {
+    const int slot = (q * NW + wave) * 64 + lane;
+    const int r = slot >> 3, c = (slot & 7) ^ ((r >> 1) & 7);
+    a_src[q] = x + (int64_t)min(m0 + r, m_rows - 1) * k_in + c * 8;
+  }
+  const int fr = lane & 31, h = lane >> 5;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  const uint32_t a_rd_row = lds_base + (wm * TM + fr) * 128;
+  uint32_t a_rd_chunk[4];
+#pragma unroll
+  for (int s4 = 0; s4 < 4; ++s4) a_rd_chunk[s4] = ((4 * h + s4) ^ ((lane >> 1) & 7)) * 16;
+
+  const uint4_t *b_src[FN];
+  const uint32_t *s_src[FN], *z_src[FN];
+#pragma unroll
+  for (int f = 0; f < FN; ++f) {
+    const int row = min(n0 + wn * TN + f * 32 + fr, n_out - 1);
+    b_src[f] = packed + (int64_t)row * (k_in >> 5) + h;
+    s_src[f] = reinterpret_cast<const uint32_t *>(scale + (int64_t)row * groups_per_row);
+    z_src[f] = reinterpret_cast<const uint32_t *>(bias + (int64_t)row * groups_per_row);
+  }
+  char *w_ring = lds + S::X_BYTES + wave * (kWStages * S::W_STAGE);
+  const uint32_t w_rd = lds_base + S::X_BYTES + wave * (kWStages * S::W_STAGE);
+
+  // Direct-to-LDS load number `op` (0 .. OPS-1) of tile `t_load` into the ring slots of tile number
+  // `t_slot`: A_OPS chunks of the x tile, FN packed fragments, FN scale and FN bias dwords.
+  // The two lanes (n, 0) and (n, 1) share one dword of scale and of bias (their groups are the
+  // same, or the two halves of it): lanes with h == 0 fetch it.
+  auto issue_op = [&](int op, int t_load, int t_slot) {
+    char *xs = lds + (t_slot % XS) * S::X_STAGE;
+    char *ws = w_ring + (t_slot % kWStages) * S::W_STAGE;
+    const int g = (t_load * 64 + h * 32) >> gs_shift;
+#pragma unroll
+    for (int q = 0; q < A_OPS; ++q)
+      if (op == q) __builtin_amdgcn_global_load_lds(a_src[q] + t_load * 64, xs + (q * NW + wave) * 1024, 16, 0, 0);
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      if (op == A_OPS + f) __builtin_amdgcn_global_load_lds(b_src[f] + t_load * 2, ws + f * 1024, 16, 0, 0);
+      if (op == A_OPS + FN + f && h == 0)
+        __builtin_amdgcn_global_load_lds(s_src[f] + (g >> 1), ws + FN * 1024 + f * 128, 4, 0, 0);
+      if (op == A_OPS + 2 * FN + f && h == 0)
+        __builtin_amdgcn_global_load_lds(z_src[f] + (g >> 1), ws + FN * 1152 + f * 128, 4, 0, 0);
+    }
+  };
+  auto issue_tile = [&](int t_load, int t_slot) {
+#pragma unroll
+    for (int op = 0; op < OPS; ++op) issue_op(op, t_load, t_slot);
+  };
+  // packed words, scale and bias dwords of tile t from this wave's ring (3 FN LDS reads)
+  auto read_weights = [&](int t, uint4_t (&wq)[FN], uint32_t (&sw)[FN], uint32_t (&zw)[FN]) {
+    const uint32_t ws = w_rd + (t % kWStages) * S::W_STAGE;
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(wq[f]) : "v"(ws + f * 1024 + lane * 16));
+      asm volatile("ds_read_b32 %0, %1" : "=v"(sw[f]) : "v"(ws + FN * 1024 + f * 128 + fr * 4));
+      asm volatile("ds_read_b32 %0, %1" : "=v"(zw[f]) : "v"(ws + FN * 1152 + f * 128 + fr * 4));
+    }
+  };
+  auto half_select = [&](int t) -> uint32_t {
+    const int g = (t * 64 + h * 32) >> gs_shift;
+    return (g & 1) ? 0x07060706u : 0x05040504u;
+  };
+
+  float16_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int f = 0; f < FN; ++f)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][f][e] = 0.f;
+
+  // ---- prologue: tiles 0 and 1 in flight, tile 0 consumed up to the B operand of its first step
+  issue_tile(0, 0);
+  issue_tile(min(1, n_tiles - 1), 1);
+  wait_vmcnt<OPS>();
+  __builtin_amdgcn_s_barrier();
+  uint4_t wq[FN], a[2][FM];
+  uint32_t sw[FN], zw[FN];
+  half2_t s2[FN], z2[FN];
+  half8_t b_cur[FN];
+  read_weights(0, wq, sw, zw);
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[0][i]) : "v"(a_rd_row + a_rd_chunk[0]), "n"(i * 4096));
+  {
+    const uint32_t sel = half_select(0);
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(wq[f]), "+v"(sw[f]), "+v"(zw[f]) : "n"(FM));
+      s2[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel));
+      z2[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel));
+      b_cur[f] = dequant_word_natural(wq[f][0], s2[f], z2[f]);
+    }
+  }
+
+  constexpr int OPS_PER_GROUP = (OPS + 3 * FM - 1) / (3 * FM);  // loads per MFMA group of steps 0..2
+  for (int t = 0; t < n_tiles; ++t) {
+    const uint32_t xs = a_rd_row + (t % XS) * S::X_STAGE;
+    const int t_ahead = min(t + 2, n_tiles - 1);  // past the end: the last tile again, into dead slots
+    // ---- steps 0..2: MFMAs of step s4, A fragments and B operand of step s4 + 1
+#pragma unroll
+    for (int s4 = 0; s4 < 3; ++s4) {
+      DequantState st[FN];
+      __builtin_amdgcn_sched_barrier(0);
+      wait_lds<0>(a[s4 & 1][FM - 1]);  // issued one step ago
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        if (i + 1 < FM) asm volatile("" : "+v"(a[s4 & 1][i]) : "v"(a[s4 & 1][FM - 1]));
+#pragma unroll
+        for (int f = 0; f < FN; ++f)
+          acc[i][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a[s4 & 1][i]), b_cur[f],
+                                                             acc[i][f], 0, 0, 0);
+        asm volatile("ds_read_b128 %0, %1 offset:%2"
+                     : "=v"(a[(s4 + 1) & 1][i])
+                     : "v"(xs + a_rd_chunk[s4 + 1]), "n"(i * 4096));
+        // one load of tile t + 2 per MFMA group: a burst of all of them right after the barrier
+        // would block every wave behind the 64 B/clk address path of the compute unit
+#pragma unroll
+        for (int o = 0; o < OPS_PER_GROUP; ++o)
+          if ((s4 * FM + i) * OPS_PER_GROUP + o < OPS) issue_op((s4 * FM + i) * OPS_PER_GROUP + o, t_ahead, t + 2);
+#pragma unroll
+        for (int f = 0; f < FN; ++f) dequant_piece<FM>(i, wq[f][s4 + 1], s2[f], z2[f], st[f]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // keep this step's fragments allocated until here: a fragment read for the next step that
+      // reused the registers of an MFMA still in flight would have to wait for that MFMA
+#pragma unroll
+      for (int i = 0; i < FM; ++i) asm volatile("" : : "v"(a[s4 & 1][i]));
+#pragma unroll
+      for (int f = 0; f < FN; ++f) b_cur[f] = dequant_result(st[f]);
+    }
+    // ---- step 3: the next tile becomes readable; its first A fragments and B operand are fetched
+    //      and built under the MFMAs of this step
+    __builtin_amdgcn_sched_barrier(0);
+    wait_lds<0>(a[1][FM - 1]);     // this wave's last LDS reads of tile t have landed (issued a step ago)
+    wait_vmcnt<OPS>();             // own loads of tile t + 1 (older than the OPS of tile t + 2)
+    __builtin_amdgcn_s_barrier();  // everybody's: tile t + 1 is readable, the x stage of tile t is dead
+    __builtin_amdgcn_sched_barrier(0);
+    uint4_t wq_next[FN];
+    read_weights(t + 1, wq_next, sw, zw);
+    const uint32_t xs_next = a_rd_row + ((t + 1) % XS) * S::X_STAGE;
+    const uint32_t sel_next = half_select(t + 1);
+    DequantState st[FN];
+    half2_t s2n[FN], z2n[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      if (i + 1 < FM) asm volatile("" : "+v"(a[1][i]) : "v"(a[1][FM - 1]));
+#pragma unroll
+      for (int f = 0; f < FN; ++f)
+        acc[i][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a[1][i]), b_cur[f], acc[i][f],
+                                                           0, 0, 0);
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[0][i]) : "v"(xs_next + a_rd_chunk[0]), "n"(i * 4096));
+      if (i == 1) {
+        // the weight reads are older than the two fragment reads issued since
+#pragma unroll
+        for (int f = 0; f < FN; ++f) {
+          asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
+          s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
+          z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+        }
+      }
+      if (i >= 2) {
+#pragma unroll
+        for (int f = 0; f < FN; ++f) dequant_piece<FM - 2>(i - 2, wq_next[f][0], s2n[f], z2n[f], st[f]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i) asm volatile("" : : "v"(a[1][i]));
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      b_cur[f] = dequant_result(st[f]);
+      wq[f] = wq_next[f];
+      s2[f] = s2n[f];
+      z2[f] = z2n[f];
+    }
+  }
+  wait_vmcnt<0>();  // surplus prefetches past the last tile
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+  // D[m][n]: lane holds n = lane % 32 and m = 8 * (e / 4) + 4 * (lane / 32) + e % 4
+  const bool interior = m0 + TILE_M <= m_rows && n0 + TILE_N <= n_out;
+#pragma unroll
+  for (int f = 0; f < FN; ++f) {
+    const int n = n0 + wn * TN + f * 32 + fr;
+    const float ob = (out_bias && n < n_out) ? (float)out_bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      half_t *dst = y + (int64_t)(m0 + wm * TM + i * 32 + 4 * h) * n_out + n;
+      if (interior) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dst[(int64_t)(8 * (e >> 2) + (e & 3)) * n_out] = (half_t)(acc[i][f][e] + ob);
+      } else if (n < n_out) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm * TM + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+          if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)(acc[i][f][e] + ob);
+        }
+      }
+    }
+  }
+}
+
+
+
+}  // namespace
+
+// (external linkage: their address is taken on the host for hipFuncSetAttribute)
+// OCC: waves per SIMD the register budget is sized for (2: 256 registers per lane, 1: 512)
+template <int WM, int WN, int FM, int FN, int XS, int OCC>
+__global__ __launch_bounds__(WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
+                                                                  const half_t *scale, const half_t *bias,
+                                                                  const half_t *out_bias, half_t *y, int n_out,
+                                                                  int k_in, int gs_shift) {
+  gemm_pipe2_body<WM, WN, FM, FN, XS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift);
+}
+
+namespace {
+
+template <int WM, int WN, int FM, int FN, int XS, int OCC>
+int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int gs_shift,
+                 hipStream_t stream) {
+  using S = Pipe2Shape<WM, WN, FM, FN, XS>;
+  constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
+  static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
+  auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC>;
+  static bool configured = false;  // same value every time: a benign race
+  if (!configured) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute(lds=%d): %s", lds_bytes, hipGetErrorString(e));
+    configured = true;
+  }
+  const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M));
+  if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_gemm_f16: m_rows=%lld too large", (long long)m_rows);
+  kern<<<grid, dim3(WM * WN * 64), lds_bytes, stream>>>(
+      reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
+      reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift);
+  return check_launch("gemm_pipe2_kernel");
+}
+
 }  // namespace
 
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
@@ -149,6 +534,22 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   if (!fast_ok || option_gemm_variant() == 1)
     return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
+  const int variant = option_gemm_variant();
+#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC) \
+  launch_pipe2<WM, WN, FM, FN, XS, OCC>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, stream)
+  // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
+  if (variant != 2 && (k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
+    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 2);
+    if (variant >= 30 && variant <= 34) shape = variant - 30;
+    switch (shape) {
+      case 0: return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
+      case 1: return GQ_PIPE2(1, 4, 8, 1, 3, 1);  // 256 x 128, 4 waves of 256 x 32
+      case 2: return GQ_PIPE2(1, 4, 4, 1, 3, 2);  // 128 x 128, 4 waves of 128 x 32, two workgroups per CU
+      case 3: return GQ_PIPE2(1, 4, 4, 2, 3, 2);  // 128 x 256, 4 waves of 128 x 64, two workgroups per CU
+      default: return GQ_PIPE2(2, 2, 4, 2, 3, 2);  // 256 x 128, 4 waves of 128 x 64
+    }
+  }
+#undef GQ_PIPE2
   const dim3 grid((unsigned)((n_out + BN - 1) / BN), (unsigned)((m_rows + BM - 1) / BM));
   if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_gemm_f16: m_rows=%lld too large", (long long)m_rows);
   gemm_tile_kernel<<<grid, dim3(256), 0, stream>>>(
