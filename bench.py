@@ -156,7 +156,7 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets)
     }
 
 
-def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384, use_graph=True):
+def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384):
     """Benchmark configuration 5: 28 layers x {4 x [4096x4096], [16384x4096], [4096x16384]} as a
     sequence of fused GEMVs, every matrix distinct (3.17 GB of packed weight in total)."""
     import torch
@@ -165,7 +165,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     g = torch.Generator(device=device)
     g.manual_seed(9)
     xs = {k: torch.randn((m_rows, k), generator=g, device=device, dtype=torch.float32).to(torch.float16) for k in (hidden, ffn)}
-    ys = {n: torch.empty((m_rows, n), dtype=torch.float16, device=device) for n in (hidden, ffn)}
+    ys = [torch.empty((m_rows, n), dtype=torch.float16, device=device) for n, _ in shapes]  # one per role
     mats = []
     seed = 1000
     for layer in range(n_layers):
@@ -178,27 +178,32 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     w_bytes = sum(n * k * (0.5 + 4.0 / GROUP) for n, k, *_ in mats)
 
     def one_pass(stream):
-        for n_out, k_in, p, s, b in mats:
+        for i, (n_out, k_in, p, s, b) in enumerate(mats):
             hip.call("gq_gemv_f16", xs[k_in].data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0,
-                     ys[n_out].data_ptr(), n_out, k_in, GROUP, stream)
+                     ys[i % 6].data_ptr(), n_out, k_in, GROUP, stream)
 
-    graph = None
-    if use_graph:
+    results = {"m": m_rows, "entries": len(mats), "weight_bytes": w_bytes}
+    # (1) one launch per matrix, replayed from a HIP graph
+    one_pass(stream_handle())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
         one_pass(stream_handle())
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            one_pass(stream_handle())
-
-    def step(_):
-        if graph is not None:
-            graph.replay()
-        else:
-            one_pass(stream_handle())
-
-    ms = time_launches(step, passes, warmup)
-    return {"m": m_rows, "launches": len(mats), "graph": bool(use_graph), "us_per_pass": ms * 1e3,
-            "weight_bytes": w_bytes, "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS}
+    ms = time_launches(lambda _: graph.replay(), passes, warmup)
+    results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                                   "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS}
+    # (2) the whole stack as one gq_gemv_sequence_f16 call.  Dependencies as in a decoder layer: the
+    # q projection waits for the previous layer, k and v share its input, then o, up and down wait
+    # for their predecessor (4 device-wide synchronisations per layer).
+    seq = hip.GemvSequence(device)
+    for i, (n_out, k_in, p, s, b) in enumerate(mats):
+        seq.add(xs[k_in], p, s, b, ys[i % 6], None, wait_previous=(i % 6) in (0, 3, 4, 5) and i > 0)
+    ms = time_launches(lambda _: seq.run(), passes, warmup)
+    torch.cuda.synchronize()
+    results["sequence"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                           "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
+                           "syncs_per_pass": sum(1 for i in range(len(mats)) if (i % 6) in (0, 3, 4, 5) and i > 0)}
+    return results
 
 
 def main():
@@ -282,7 +287,9 @@ def main():
         for m in (1, 4):
             r = bench_stack(hip, device, m, passes=20, warmup=3)
             extra["stack"].append(r)
-            log(f"  stack m={m}: {r['us_per_pass']:.0f} us/pass, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
+            for mode in ("per_launch_graph", "sequence"):
+                log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
+                    f"({r[mode]['hbm_frac']:.1%})")
             torch.cuda.empty_cache()
     extra["bench_wall_s"] = round(time.time() - t_begin, 1)
 

@@ -17,10 +17,8 @@
  *     (nothing was launched); a positive value is a `hipError_t` from the runtime.
  *     `gq_last_error()` returns a thread-local, human-readable description of the last
  *     non-zero return on the calling thread.
- *   - Functions are re-entrant and keep no per-call state; the split-K workspace of the
- *     matmul entry points is per device and protected per stream by stream order only:
- *     two matmul calls running concurrently on different streams of one device must not
- *     both use split-K shapes (see gq_linear_f16).
+ *   - Functions are re-entrant, allocate nothing and keep no per-call state (one exception:
+ *     gq_gemv_sequence_f16, see there); every entry point can be captured in a HIP graph.
  *
  * Packed layout (group_quantize_decompress.py:127-135, group_quantize_decompress_codelet.cpp:11-14)
  *   packed[r][g][i] is a little-endian uint16 holding four 4-bit codes, most significant
@@ -99,10 +97,9 @@ int gq_decompress_f16_transposed(const uint16_t *packed, const uint16_t *scale, 
  * gq_gemm_f16  prefill-sized batches (any m_rows >= 1; built for m_rows >= 16).
  * gq_linear_f16 picks between them by m_rows; it is what the LinearGQ wrapper calls.
  *
- * Shapes with k_in > 4096 are split along K over several workgroups that meet in a
- * per-device workspace owned by the library: calls on ONE stream are ordered and safe;
- * concurrent calls of such shapes on different streams of the same device are not.
- * Requirements: group_size % 4 == 0, k_in % group_size == 0.
+ * Requirements: group_size % 4 == 0, k_in % group_size == 0.  Fast kernels need a power-of-two
+ * group_size >= 32, k_in % 128 == 0 (GEMV) or % 64 == 0 (GEMM) and 16-byte aligned x / packed;
+ * other shapes run slower generic kernels with the same results.
  */
 int gq_gemv_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
@@ -115,6 +112,41 @@ int gq_gemm_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                   const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                   int64_t k_in, int64_t group_size, void *stream);
+
+/*
+ * A sequence of decode GEMVs (a layer stack) as one call.  No counterpart in the reference, where
+ * a model is a chain of LinearGQ.build calls (popxl_addons/layers/linear_gq.py:99-109) compiled
+ * into one static device program; this entry point is the analogue for a chain of gq_gemv_f16
+ * calls: entry i computes exactly what gq_gemv_f16 would, entries run in order, and an entry with
+ * wait_previous != 0 starts only after every earlier entry has completed (set it when x or
+ * out_bias of the entry is produced by an earlier one).  Entries without the flag may overlap
+ * earlier ones.
+ *
+ * For group_size 64, k_in % 512 == 0, m_rows <= 8 and 16-byte aligned pointers the whole sequence
+ * runs as one persistent kernel (one workgroup per compute unit) that streams the packed weights
+ * without a gap between entries; any other sequence runs as one launch per entry.
+ *
+ *   descs         host copy of the entries (validated here, not read after the call returns)
+ *   descs_device  device copy of the same `count` entries (read by the kernel)
+ *   status        device int32 or NULL; set to 1 if the kernel gave up waiting for earlier entries
+ *                 (it then still terminates; results are invalid).  The caller zeroes it.
+ * The persistent kernel keeps its progress counters in device globals: at most one sequence may
+ * run on a device at a time.
+ */
+typedef struct gq_gemv_desc {
+  const uint16_t *x;        /* [m_rows, k_in] binary16 */
+  const uint16_t *packed;   /* [n_out, k_in / group_size, group_size / 4] */
+  const uint16_t *scale;    /* [n_out, k_in / group_size] binary16 */
+  const uint16_t *bias;     /* [n_out, k_in / group_size] binary16 */
+  const uint16_t *out_bias; /* [n_out] binary16 or NULL */
+  uint16_t *y;              /* [m_rows, n_out] binary16 */
+  int32_t m_rows, n_out, k_in, group_size;
+  int32_t wait_previous;
+  int32_t reserved;         /* 0 */
+} gq_gemv_desc;
+
+int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                         int32_t *status, void *stream);
 
 /*
  * Device-side compress for binary16 input: bit-identical packed/scale/bias to

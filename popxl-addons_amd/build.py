@@ -18,7 +18,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libgq_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["gq_api.hip", "gq_decompress.hip", "gq_compress.hip", "gq_gemv.hip", "gq_gemm.hip"]
+SOURCES = ["gq_api.hip", "gq_decompress.hip", "gq_compress.hip", "gq_gemv.hip", "gq_gemv_stream.hip", "gq_gemm.hip"]
 
 # -ffp-contract=off: the decompress contract is "fp16 multiply, then fp16 add" (two roundings);
 # kernels that want an fma ask for one explicitly.  Packed-fp32 instruction selection is disabled.

@@ -143,6 +143,27 @@ int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, con
                          (hipStream_t)stream);
 }
 
+int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                         int32_t *status, void *stream) {
+  if (count < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: negative count");
+  if (count == 0) return GQ_OK;
+  if (!descs || !descs_device) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_sequence_f16: descs is NULL");
+  if (gq::misaligned(descs_device, 8) || gq::misaligned(status, 4))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_f16: misaligned descs_device or status");
+  for (int64_t i = 0; i < count; ++i) {
+    const gq_gemv_desc &d = descs[i];
+    const int rc = gq::check_linear_args("gq_gemv_sequence_f16", d.x, d.m_rows, d.packed, d.scale, d.bias,
+                                         d.out_bias, d.y, d.n_out, d.k_in, d.group_size);
+    if (rc < 0) return rc;
+    if (rc == 0 || d.k_in == 0)
+      return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld is empty", (long long)i);
+    if (d.m_rows > 16)
+      return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld has m_rows=%d > 16", (long long)i,
+                      d.m_rows);
+  }
+  return gq::launch_gemv_sequence(descs, descs_device, count, status, (hipStream_t)stream);
+}
+
 int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,
                     int32_t *nonfinite_flag, int64_t rows, int64_t n_groups, int64_t group_size,
                     void *stream) {

@@ -34,6 +34,8 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, hipStream_t stream);
+int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
+                         hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
                     int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
 

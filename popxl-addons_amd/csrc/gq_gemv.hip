@@ -5,11 +5,11 @@
 // writing the fp16 weight to memory.  HBM-bound on the packed weight: 0.5 + 4/gs bytes per
 // weight element.
 #include "gq_common.h"
+#include "gq_gemv_dequant.h"
 
 namespace gq {
 namespace {
 
-__device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 
 // ---------------------------------------------------------------------------------------
 // MFMA path.  v_mfma_f32_16x16x32_f16 computes D[16x16] += A[16x32] * B[32x16]; here A holds
@@ -22,46 +22,6 @@ __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_c
 // A wave owns 16 rows and walks K in chunks of 512 (four 16-byte loads per lane); the waves of
 // a workgroup take interleaved chunks of the same 16 rows and their partial sums meet in LDS.
 // ---------------------------------------------------------------------------------------
-
-// (w & mask) | magic in one VALU op; mask and magic live in VGPRs (one constant-bus operand is
-// all a VOP3 instruction may take on this target).
-__device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "v"(mask), "v"(magic));
-  return r;
-}
-
-// 8 codes of `w` -> 8 fp16 weights, order (0,4,1,5,2,6,3,7).  The nibble is or-ed into the
-// mantissa of 1024.0 (ulp 1) or, for nibbles sitting at bits 7:4, read as 1024 + 16*code; both
-// are brought back to the exact code with one packed op, then scaled with a packed fma:
-// 13 VALU instructions per 8 weights.
-__device__ __forceinline__ half8_t dequant_word(uint32_t w, half2_t s2, half2_t b2) {
-  const half2_t kNeg1024 = {(half_t)-1024.0f, (half_t)-1024.0f};
-  const half2_t kSixteenth = {(half_t)0.0625f, (half_t)0.0625f};
-  const half2_t kNeg64 = {(half_t)-64.0f, (half_t)-64.0f};
-  const uint32_t kLo = 0x000F000Fu, kHi = 0x00F000F0u, kMagic = 0x64006400u;
-  const uint32_t hi = w >> 8;
-  const half2_t c0 = __builtin_elementwise_fma(as_half2(and_or(hi, kHi, kMagic)), kSixteenth, kNeg64);
-  const half2_t c1 = as_half2(and_or(hi, kLo, kMagic)) + kNeg1024;
-  const half2_t c2 = __builtin_elementwise_fma(as_half2(and_or(w, kHi, kMagic)), kSixteenth, kNeg64);
-  const half2_t c3 = as_half2(and_or(w, kLo, kMagic)) + kNeg1024;
-  const half2_t w0 = __builtin_elementwise_fma(c0, s2, b2);
-  const half2_t w1 = __builtin_elementwise_fma(c1, s2, b2);
-  const half2_t w2 = __builtin_elementwise_fma(c2, s2, b2);
-  const half2_t w3 = __builtin_elementwise_fma(c3, s2, b2);
-  return __builtin_shufflevector(__builtin_shufflevector(w0, w1, 0, 1, 2, 3),
-                                 __builtin_shufflevector(w2, w3, 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
-// 8 consecutive fp16 of x -> order (0,4,1,5,2,6,3,7)
-__device__ __forceinline__ half8_t permute_x(uint4_t q) {
-  uint4_t p;
-  p.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);
-  p.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);
-  p.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);
-  p.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);
-  return __builtin_bit_cast(half8_t, p);
-}
 
 // One chunk = 512 contraction indices = four 16-byte loads per lane and row block ("slots" of
 // 128 indices: lane (r, kc) takes bytes [64 * slot + 16 * kc, +16) of its row's chunk).

@@ -27,6 +27,7 @@ EXPORTS = (
     "gq_gemv_f16",
     "gq_gemm_f16",
     "gq_linear_f16",
+    "gq_gemv_sequence_f16",
     "gq_compress_f16",
 )
 
@@ -74,6 +75,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, p]
         fn.restype = ctypes.c_int
+    lib.gq_gemv_sequence_f16.argtypes = [p, p, i64, p, p]
+    lib.gq_gemv_sequence_f16.restype = ctypes.c_int
     lib.gq_compress_f16.argtypes = [p, p, p, p, p, i64, i64, i64, p]
     lib.gq_compress_f16.restype = ctypes.c_int
     if lib.gq_abi_version() != GQ_ABI_VERSION:
@@ -96,3 +99,64 @@ def call(name, *args):
 
 def set_option(name, value):
     call("gq_set_option", name.encode(), int(value))
+
+
+class GemvSequence:
+    """A list of decode GEMVs run by one `gq_gemv_sequence_f16` call (see include/gq_hip.h).
+
+    add(x, packed, scale, bias, y, out_bias=None, wait_previous=False) appends an entry from torch
+    tensors on the GPU (kept alive by this object); run() enqueues the whole list on the current
+    stream.  `status` is a device int32 the kernel sets to 1 if it gave up waiting.
+    """
+
+    def __init__(self, device):
+        import numpy as np
+
+        self.device = device
+        self.dtype = np.dtype(
+            [("x", "<u8"), ("packed", "<u8"), ("scale", "<u8"), ("bias", "<u8"), ("out_bias", "<u8"), ("y", "<u8"),
+             ("m_rows", "<i4"), ("n_out", "<i4"), ("k_in", "<i4"), ("group_size", "<i4"), ("wait_previous", "<i4"),
+             ("reserved", "<i4")]
+        )
+        assert self.dtype.itemsize == 72  # sizeof(gq_gemv_desc)
+        self.entries = []
+        self.keep = []
+        self._host = None
+        self._dev = None
+        self.status = None
+
+    def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False):
+        m_rows, k_in = x.shape
+        n_out, n_groups, n_ids = packed.shape
+        assert y.shape == (m_rows, n_out) and n_groups * n_ids * 4 == k_in
+        for t in (x, packed, scale, bias, y):
+            assert t.is_cuda and t.is_contiguous()
+        self.entries.append(
+            (x.data_ptr(), packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+             0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, n_ids * 4,
+             1 if wait_previous else 0, 0)
+        )
+        self.keep.append((x, packed, scale, bias, y, out_bias))
+        self._host = None
+
+    def _finalise(self):
+        import numpy as np
+        import torch
+
+        self._host = np.array(self.entries, dtype=self.dtype)
+        self._dev = torch.from_numpy(self._host.view(np.uint8).copy()).to(self.device)
+        self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
+
+    def run(self):
+        import torch
+
+        if self._host is None:
+            self._finalise()
+        call(
+            "gq_gemv_sequence_f16",
+            self._host.ctypes.data,
+            self._dev.data_ptr(),
+            len(self.entries),
+            self.status.data_ptr(),
+            torch.cuda.current_stream(self.device).cuda_stream,
+        )

@@ -146,3 +146,111 @@ def test_linearity_at_full_size(hip, device):
         torch.cuda.synchronize()
         err = (ys[2] - ys[0] - ys[1]).abs().max().item() / ys[2].abs().max().item()
         assert err <= TOL, (entry, err)
+
+
+def _sequence_case(hip, device, oracle, shapes, m_rows, chained, seed=50):
+    """Entries of the given (n_out, k_in) shapes; `chained`: entry i reads entry i-1's output."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    rng = np.random.default_rng(seed)
+    seq = GemvSequence(device)
+    refs, outs = [], []
+    x_host = activations(m_rows, shapes[0][1], seed)
+    x_dev = to_dev(x_host, device)
+    for i, (n_out, k_in) in enumerate(shapes):
+        # a weight scale that keeps a chain of layers at unit magnitude
+        w = (rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in))).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        ob = rng.normal(0, 0.1, (n_out,)).astype(np.float16) if i % 2 else None
+        w_dec = oracle.np_decompress(packed, scale, bias)
+        if chained and i > 0:
+            assert k_in == shapes[i - 1][0]
+            x_host = refs[-1].astype(np.float16)  # what the device chain holds up to fp16 rounding
+            x_in = outs[-1]
+        else:
+            x_host = activations(m_rows, k_in, seed + i)
+            x_in = to_dev(x_host, device)
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        seq.add(x_in, to_dev(packed, device), to_dev(scale, device), to_dev(bias, device), y,
+                None if ob is None else to_dev(ob, device), wait_previous=chained and i > 0)
+        refs.append(oracle.np_linear(x_host, w_dec, ob))
+        outs.append(y)
+    return seq, refs, outs
+
+
+@pytest.mark.parametrize("m_rows", [1, 4, 8])
+def test_gemv_sequence_independent_entries(hip, device, oracle, m_rows):
+    """Every entry of a sequence equals the single-call result (benchmark configuration 5 shapes,
+    ragged row counts, a k_in that is not a multiple of 4096)."""
+    shapes = [(4096, 4096), (4096, 4096), (1000, 4096), (16384, 4096), (4096, 16384), (16, 512), (5000, 1536), (40, 8192)]
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, m_rows, chained=False)
+    for _ in range(2):  # twice: the progress counters must be back at zero after a run
+        for y in outs:
+            y.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        for (n_out, k_in), y, ref in zip(shapes, outs, refs):
+            yy = y.cpu().numpy()
+            assert np.isfinite(yy).all(), (n_out, k_in)
+            assert normalised_error(yy, ref) <= TOL, (n_out, k_in)
+
+
+@pytest.mark.parametrize("m_rows", [1, 4])
+def test_gemv_sequence_chained_entries(hip, device, oracle, m_rows):
+    """wait_previous: each entry consumes the previous entry's output (other compute units wrote it)."""
+    shapes = [(4096, 4096), (2048, 4096), (4096, 2048), (16384, 4096), (4096, 16384), (512, 4096)]
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, m_rows, chained=True)
+    for _ in range(3):
+        for y in outs:
+            y.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        # compare link by link: reference of entry i is computed from the DEVICE output of entry i-1
+        x_prev = None
+        for i, ((n_out, k_in), y) in enumerate(zip(shapes, outs)):
+            yy = y.cpu().numpy()
+            assert np.isfinite(yy).all(), i
+            if i == 0:
+                assert normalised_error(yy, refs[0]) <= TOL
+            else:
+                e = seq.keep[i]
+                w_dec = oracle.np_decompress(e[1].cpu().numpy(), e[2].cpu().numpy(), e[3].cpu().numpy())
+                ob = None if e[5] is None else e[5].cpu().numpy()
+                assert normalised_error(yy, oracle.np_linear(x_prev, w_dec, ob)) <= TOL, i
+            x_prev = yy
+
+
+def test_gemv_sequence_fallback_and_graph(hip, device, oracle):
+    """Shapes outside the persistent kernel (group 32) run entry by entry; the persistent kernel
+    replays correctly from a captured graph."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    rng = np.random.default_rng(3)
+    seq = GemvSequence(device)
+    w = rng.normal(0, 0.02, (96, 256)).astype(np.float16)
+    packed, scale, bias = group_quantize_compress_numpy(w, 32)
+    x = activations(2, 256, 1)
+    y = torch.empty((2, 96), dtype=torch.float16, device=device)
+    seq.add(to_dev(x, device), to_dev(packed, device), to_dev(scale, device), to_dev(bias, device), y)
+    seq.run()
+    torch.cuda.synchronize()
+    assert normalised_error(y.cpu().numpy(), oracle.np_linear(x, oracle.np_decompress(packed, scale, bias))) <= TOL
+
+    shapes = [(4096, 4096), (4096, 4096), (1024, 4096)]
+    seq2, refs, outs = _sequence_case(hip, device, oracle, shapes, 1, chained=True, seed=60)
+    seq2.run()
+    torch.cuda.synchronize()
+    want = [o.clone() for o in outs]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        seq2.run()
+    for _ in range(3):
+        for o in outs:
+            o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(seq2.status.item()) == 0
+        for o, w_ in zip(outs, want):
+            assert torch.equal(o, w_)
