@@ -21,15 +21,20 @@
 namespace gq {
 namespace {
 
-constexpr int kWaves = 8, kThreads = kWaves * 64;
+constexpr int kWaves = 8;                         // compute waves
+constexpr int kThreadsAll = (kWaves + 2) * 64;    // + reducer + poller
 constexpr int kItemBytes = 4096 + 512;  // packed words, 16 rows x 16 B of scale, 16 rows x 16 B of bias
 constexpr int kItemOps = 5;             // direct-to-LDS loads per item: 4 packed + 1 scale/bias
 constexpr int kPassRows = 4;            // row blocks per pass (accumulators held by a wave)
 constexpr unsigned kSpinLimit = 1u << 18;
 
-// progress of the running sequence on this device; the last workgroup to leave resets them
-__device__ unsigned int g_arrived;  // (workgroup, entry) completions
-__device__ unsigned int g_exited;   // workgroups that left the kernel
+// Progress of the running sequence on this device.  Every workgroup publishes the number of
+// entries it has completed in its own word (plain device-scope stores: 256 read-modify-writes of
+// one counter per entry would serialise at the memory side); the last workgroup to leave the
+// kernel clears the words.
+constexpr int kMaxGroups = 1024;
+__device__ __attribute__((aligned(16))) unsigned int g_progress[kMaxGroups];
+__device__ unsigned int g_exited;  // workgroups that left the kernel
 
 struct Entry {  // = gq_gemv_desc
   const half_t *x;
@@ -52,46 +57,217 @@ struct Cursor {
   int d, pass, phase, j;  // entry, pass of 4 row blocks, phase of 4096 indices, row block in pass
 };
 
-// MCAP: largest batch the x stage of a wave holds (KiB); NS: depth of the weight ring.
+// what the kernel needs of an entry, kept in LDS: descriptor reads from global memory in the
+// work loop cost microseconds each
+struct CachedEntry {
+  const uint4_t *packed;
+  const half_t *scale, *bias, *x, *out_bias;
+  half_t *y;
+  int n_out, k_in;
+  short m_rows, wait_previous;
+  int nrb;  // row blocks owned by this workgroup
+};
+static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
+constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
+
+// cache policy of a direct-to-LDS load: sc0 | sc1 = coherent at device scope (bypasses the L1 of
+// the compute unit and the non-coherent part of the L2 of its XCD)
+constexpr int kAuxDeviceCoherent = (1 << 0) | (1 << 4);
+
+// LDS words shared by the waves of a workgroup
+struct Control {
+  unsigned deposited;  // mailbox deposits so far (8 per pass)
+  unsigned consumed;   // passes whose mailboxes the reducer has read
+  unsigned ready;      // entries known to be complete on the whole device
+  unsigned failed;     // the poller gave up
+};
+
+__device__ __forceinline__ unsigned lds_load(const unsigned *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// MCAP: largest batch (the x stage of a wave holds MCAP KiB); NS: depth of the weight ring.
 // (A __device__ function: a __global__ template is also instantiated for the host, where the
 // target builtins and inline assembly do not exist.)
+//
+// Waves 0..7 compute; they never meet at a workgroup barrier.  After the last chunk of a pass a
+// wave drops its 16 x m partial sums into its mailbox and goes on with the next pass or entry.
+// Wave 8, the reducer, adds the eight mailboxes in a fixed order, stores y and counts the
+// workgroup as arrived for the entry.  Wave 9, the poller, watches the device-wide arrival count
+// and publishes in LDS how many entries are complete; a compute wave that needs an earlier result
+// waits for that number only.
+//
+// Visibility of results between compute units needs no cache flush: y is written with device-scope
+// stores (sc1, write-through to the coherent level), the reducer waits for its stores before it
+// counts, and x is read with device-coherent loads.
 template <int MCAP, int NS>
 __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries,
                                                  int *__restrict__ status) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int kWaveBytes = NS * kItemBytes + MCAP * 1024;
+  constexpr int kMailBytes = kPassRows * 4 * MCAP * 16;  // per wave: [row block][kc][m] float4
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kc = lane >> 4;
   const int G = gridDim.x, b = blockIdx.x;
+  CachedEntry *cache = reinterpret_cast<CachedEntry *>(lds + kWaves * kWaveBytes);
+  char *mail = lds + kWaves * kWaveBytes + kMaxEntries * 64;
+  Control *ctl = reinterpret_cast<Control *>(mail + kWaves * kMailBytes);
+
+  for (int i = tid; i < n_entries; i += kThreadsAll) {
+    const Entry e = entries[i];
+    CachedEntry c;
+    c.packed = e.packed;
+    c.scale = e.scale;
+    c.bias = e.bias;
+    c.x = e.x;
+    c.out_bias = e.out_bias;
+    c.y = e.y;
+    c.n_out = e.n_out;
+    c.k_in = e.k_in;
+    c.m_rows = (short)e.m_rows;
+    c.wait_previous = (short)(e.wait_previous != 0);
+    const int rb = (e.n_out + 15) >> 4;
+    c.nrb = rb > b ? (rb - b + G - 1) / G : 0;
+    cache[i] = c;
+  }
+  if (tid == 0) *ctl = Control{0u, 0u, 0u, 0u};
+  __syncthreads();  // the only workgroup barrier
+
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+
+  // ============================================================================ poller
+  if (wave == kWaves + 1) {
+    int last_waited = 0;
+    for (int d = 1; d < n_entries; ++d)
+      if (cache[d].wait_previous) last_waited = d;
+    // one 16-byte device-coherent load per lane covers 256 workgroups; the minimum over all of them
+    // is the number of entries complete everywhere
+    unsigned ready = 0, spins = 0;
+    const int rounds = (G + 255) >> 8;
+    while (ready < (unsigned)last_waited) {
+      unsigned lo = 0xffffffffu;
+      for (int k = 0; k < rounds; ++k) {
+        const int first = (k * 64 + lane) * 4;
+        uint4_t v;
+        asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+                     : "=v"(v)
+                     : "v"(g_progress + first)
+                     : "memory");
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (first + i < G) lo = min(lo, v[i]);
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) lo = min(lo, (unsigned)__shfl_xor((int)lo, off, 64));
+      if (lo > ready) {
+        ready = lo;
+        if (lane == 0) __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        spins = 0;
+      } else if (++spins > kSpinLimit) {  // some workgroup is not running: give up, let everybody finish
+        if (lane == 0) {
+          __hip_atomic_store(&ctl->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (status) atomicExch(status, 1);
+        }
+        break;
+      }
+    }
+    return;
+  }
+
+  // =========================================================================== reducer
+  if (wave == kWaves) {
+    unsigned q = 0;  // passes reduced so far
+    for (int d = 0; d < n_entries; ++d) {
+      const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), n_out = uni(cache[d].n_out);
+      half_t *y = cache[d].y;
+      const half_t *out_bias = cache[d].out_bias;
+      for (int pass = 0; pass * kPassRows < nrb; ++pass, ++q) {
+        const int nj = min(kPassRows, nrb - pass * kPassRows);
+        while (lds_load(&ctl->deposited) < (q + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
+        // lane -> (row block j, kc, m): 16 lanes per row block when MCAP == 4
+        for (int t = lane; t < nj * 4 * MCAP; t += 64) {
+          const int m = t % MCAP, kq = (t / MCAP) & 3, j = t / (4 * MCAP);
+          float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int w = 0; w < kWaves; ++w) sum += *reinterpret_cast<const float4_t *>(mail + w * kMailBytes + t * 16);
+          if (m < m_rows) {
+            const int n0 = (b + (pass * kPassRows + j) * G) * 16 + 4 * kq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int n = n0 + i;
+              if (n < n_out) {
+                float v = sum[i];
+                if (out_bias) v += (float)out_bias[n];
+                const half_t hv = (half_t)v;
+                // device-scope store: written through to where every compute unit reads it
+                __hip_atomic_store(reinterpret_cast<unsigned short *>(y) + (int64_t)m * n_out + n,
+                                   __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+            }
+          }
+        }
+        // the mailboxes have been read (the sums above depend on them): free them
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_store(&ctl->consumed, q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      wait_vm<0>();  // every lane's stores of this entry are complete ...
+      if (lane == 0)   // ... then publish
+        __hip_atomic_store(&g_progress[b], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // the last workgroup out clears the progress words: by then every poller has seen all it needs
+    wait_vm<0>();  // this workgroup's last progress word is in memory before it counts itself out
+    unsigned last = 0;
+    if (lane == 0) last = atomicAdd(&g_exited, 1u) == (unsigned)G - 1;
+    if (__builtin_amdgcn_readfirstlane((int)last)) {
+      wait_vm<0>();
+      for (int i = lane; i < G; i += 64) __hip_atomic_store(&g_progress[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
+
+  // ==================================================================== compute waves
   char *ring = lds + wave * kWaveBytes;
   char *xstage = ring + NS * kItemBytes;
   const uint32_t ring_rd = (uint32_t)(uintptr_t)ring, x_rd = (uint32_t)(uintptr_t)xstage;
   const uint32_t half_sel = (kc & 2) ? 0x07060706u : 0x05040504u;  // lane's group within a slot: kc / 2
 
-  // number of row blocks this workgroup owns in entry e
-  auto my_row_blocks = [&](const Entry &e) {
-    const int rb = (e.n_out + 15) >> 4;
-    return rb > b ? (rb - b + G - 1) / G : 0;
+  // The producer walks the same item list as the consumer, NS items ahead.  Its entry is held in
+  // scalar registers (values read from LDS are made wave-uniform explicitly), so that advancing
+  // the cursor is a handful of scalar instructions.
+  auto uni_ptr = [&](const void *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    return (const char *)(uintptr_t)(((uint64_t)(uint32_t)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v));
+  };
+  struct ProducerEntry {
+    const char *packed, *scale, *bias;
+    int n_out, k_in, nrb, phases;
+  } pe = {nullptr, nullptr, nullptr, 1, 512, 0, 1};
+  auto load_producer_entry = [&](int d) {
+    if (d >= n_entries) return;
+    pe.packed = uni_ptr(cache[d].packed);
+    pe.scale = uni_ptr(cache[d].scale);
+    pe.bias = uni_ptr(cache[d].bias);
+    pe.n_out = uni(cache[d].n_out);
+    pe.k_in = uni(cache[d].k_in);
+    pe.nrb = uni(cache[d].nrb);
+    pe.phases = (pe.k_in + 4095) >> 12;
   };
   // does cursor c name a work item of this wave?  (entries without rows for this workgroup and
   // chunks past k_in are skipped)
   auto valid = [&](const Cursor &c) {
     if (c.d >= n_entries) return true;  // the end is a valid resting place
-    const Entry &e = entries[c.d];
-    const int nrb = my_row_blocks(e);
-    return c.pass * kPassRows + c.j < nrb && (c.phase * kWaves + wave) * 512 < e.k_in;
+    return c.pass * kPassRows + c.j < pe.nrb && (c.phase * kWaves + wave) * 512 < pe.k_in;
   };
   auto step = [&](Cursor &c) {
-    const Entry &e = entries[c.d];
-    const int nrb = my_row_blocks(e);
-    const int phases = (e.k_in + 4095) >> 12;
-    if (++c.j < kPassRows && c.pass * kPassRows + c.j < nrb) return;
+    if (++c.j < kPassRows && c.pass * kPassRows + c.j < pe.nrb) return;
     c.j = 0;
-    if (++c.phase < phases) return;
+    if (++c.phase < pe.phases) return;
     c.phase = 0;
-    if (++c.pass * kPassRows < nrb) return;
+    if (++c.pass * kPassRows < pe.nrb) return;
     c.pass = 0;
     ++c.d;
+    load_producer_entry(c.d);
   };
   auto next_item = [&](Cursor &c) {
     do step(c);
@@ -99,22 +275,22 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   };
   // direct-to-LDS loads of the item at cursor c into ring slot `slot`
   auto issue_item = [&](const Cursor &c, int slot) {
-    const Entry &e = entries[c.d];
     const int rb = b + (c.pass * kPassRows + c.j) * G;
-    const int row = min(rb * 16 + r, e.n_out - 1);
+    const int row = min(rb * 16 + r, pe.n_out - 1);
     const int chunk = c.phase * kWaves + wave;
     char *dst = ring + slot * kItemBytes;
-    const uint4_t *src = e.packed + (int64_t)row * (e.k_in >> 5) + chunk * 16 + kc;
+    const uint4_t *src = reinterpret_cast<const uint4_t *>(pe.packed) + (int64_t)row * (pe.k_in >> 5) + chunk * 16 + kc;
 #pragma unroll
     for (int s = 0; s < 4; ++s) __builtin_amdgcn_global_load_lds(src + s * 4, dst + s * 1024, 16, 0, 0);
     // lanes kc == 0 fetch the 8 scales of their row's chunk, lanes kc == 1 the 8 biases
     if (kc < 2) {
-      const half_t *sb = (kc == 0 ? e.scale : e.bias) + (int64_t)row * (e.k_in >> 6) + chunk * 8;
+      const half_t *sb = reinterpret_cast<const half_t *>(kc == 0 ? pe.scale : pe.bias) + (int64_t)row * (pe.k_in >> 6) + chunk * 8;
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(sb), dst + 4096, 16, 0, 0);
     }
   };
 
   Cursor prod = {0, 0, 0, 0};  // the producer's position: first item of this wave
+  load_producer_entry(0);
   if (n_entries > 0 && !valid(prod)) next_item(prod);
   int n_ahead = 0;  // items issued and not yet consumed
   while (n_ahead < NS && prod.d < n_entries) {
@@ -122,61 +298,49 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     ++n_ahead;
     next_item(prod);
   }
-  int slot = 0;  // ring slot of the consumer's item
-  bool failed = false;
+  int slot = 0;    // ring slot of the consumer's item
+  unsigned q = 0;  // passes finished so far (same count in every wave)
 
   half8_t xp[4][4];
   const half_t *x_loaded = nullptr;  // x fragments in registers belong to (x_loaded, chunk x_chunk)
   int x_chunk = -1, x_k = 0, x_m = 0;
 
   for (int d = 0; d < n_entries; ++d) {
-    const Entry e = entries[d];
-    const int nrb = my_row_blocks(e);
-    const int phases = (e.k_in + 4095) >> 12;
-    if (e.wait_previous && d > 0) {
-      // every workgroup has finished every earlier entry
-      if (tid == 0) {
-        const unsigned target = (unsigned)d * (unsigned)G;
-        unsigned spins = 0;
-        while (!failed && __hip_atomic_load(&g_arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-          __builtin_amdgcn_s_sleep(2);
-          if (++spins > kSpinLimit) {
-            failed = true;
-            if (status) atomicExch(status, 1);
-          }
-        }
-        __threadfence();  // acquire: earlier entries' y becomes visible to this compute unit
-      }
-      __syncthreads();
+    const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), k_in = uni(cache[d].k_in);
+    const half_t *x = reinterpret_cast<const half_t *>(uni_ptr(cache[d].x));
+    const int phases = (k_in + 4095) >> 12;
+    if (uni(cache[d].wait_previous) && d > 0) {
+      // every workgroup has finished every earlier entry (published by the poller)
+      while (lds_load(&ctl->ready) < (unsigned)d && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
       x_loaded = nullptr;
     }
-    for (int pass = 0; pass * kPassRows < nrb; ++pass) {
+    for (int pass = 0; pass * kPassRows < nrb; ++pass, ++q) {
       const int nj = min(kPassRows, nrb - pass * kPassRows);
       float4_t acc[kPassRows];
 #pragma unroll
       for (int j = 0; j < kPassRows; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
       for (int phase = 0; phase < phases; ++phase) {
         const int chunk = phase * kWaves + wave;
-        if (chunk * 512 >= e.k_in) continue;
+        if (chunk * 512 >= k_in) continue;
         // ---- x fragments of this chunk (kept when the previous entry used the same ones)
-        const bool reload_x = !(x_loaded == e.x && x_chunk == chunk && x_k == e.k_in && x_m == e.m_rows);
+        const bool reload_x = !(x_loaded == x && x_chunk == chunk && x_k == k_in && x_m == m_rows);
         if (reload_x) {
-          for (int m = 0; m < e.m_rows; ++m)
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(e.x + (int64_t)m * e.k_in + chunk * 512) + lane,
-                                             xstage + m * 1024, 16, 0, 0);
+          for (int m = 0; m < m_rows; ++m)
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
+                                             xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
           wait_vm<0>();  // x is the youngest load: everything in flight lands with it
-          uint4_t q[4][4];
+          uint4_t xq[4][4];
 #pragma unroll
           for (int j4 = 0; j4 < 4; ++j4)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) q[j4][s] = uint4_t{0u, 0u, 0u, 0u};
-          if (r < e.m_rows) {
+            for (int s = 0; s < 4; ++s) xq[j4][s] = uint4_t{0u, 0u, 0u, 0u};
+          if (r < m_rows) {
 #pragma unroll
             for (int j4 = 0; j4 < 4; ++j4)
 #pragma unroll
               for (int s = 0; s < 4; ++s)
                 asm volatile("ds_read_b128 %0, %1 offset:%2"
-                             : "=v"(q[j4][s])
+                             : "=v"(xq[j4][s])
                              : "v"(x_rd + r * 1024 + kc * 64), "n"((j4 * 16 + s) * 16));
           }
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -184,13 +348,13 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           for (int j4 = 0; j4 < 4; ++j4)
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-              asm volatile("" : "+v"(q[j4][s]));  // consumed after the wait
-              xp[j4][s] = permute_x(q[j4][s]);
+              asm volatile("" : "+v"(xq[j4][s]));  // consumed after the wait
+              xp[j4][s] = permute_x(xq[j4][s]);
             }
-          x_loaded = e.x;
+          x_loaded = x;
           x_chunk = chunk;
-          x_k = e.k_in;
-          x_m = e.m_rows;
+          x_k = k_in;
+          x_m = m_rows;
         }
 #pragma unroll
         for (int j = 0; j < kPassRows; ++j) {
@@ -228,53 +392,25 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           }
         }
       }
-      // ---- partial sums of the 8 waves meet in LDS.  Each wave's x stage doubles as its mailbox:
-      //      the fragments it held are in registers by now.
+      // ---- drop the partial sums into this wave's mailbox once the reducer has emptied it
+      while (lds_load(&ctl->consumed) < q) __builtin_amdgcn_s_sleep(1);
+      if (r < MCAP) {
 #pragma unroll
-      for (int j = 0; j < kPassRows; ++j)
-        if (j < nj) *reinterpret_cast<float4_t *>(xstage + j * 1024 + lane * 16) = acc[j];
-      __syncthreads();
-      for (int t = tid; t < nj * 64; t += kThreads) {
-        const int j = t >> 6, l = t & 63;
-        float4_t sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) sum += *reinterpret_cast<const float4_t *>(lds + w * kWaveBytes + NS * kItemBytes + j * 1024 + l * 16);
-        const int m = l & 15;
-        if (m < e.m_rows) {
-          const int n0 = (b + (pass * kPassRows + j) * G) * 16 + 4 * (l >> 4);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int n = n0 + i;
-            if (n < e.n_out) {
-              float v = sum[i];
-              if (e.out_bias) v += (float)e.out_bias[n];
-              e.y[(int64_t)m * e.n_out + n] = (half_t)v;
-            }
-          }
-        }
+        for (int j = 0; j < kPassRows; ++j)
+          if (j < nj) *reinterpret_cast<float4_t *>(mail + wave * kMailBytes + ((j * 4 + kc) * MCAP + r) * 16) = acc[j];
       }
-      __syncthreads();
-    }
-    // ---- this workgroup is done with entry d
-    if (tid == 0) {
-      __threadfence();  // release: y is visible device-wide before the count
-      atomicAdd(&g_arrived, 1u);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the deposit is in LDS before it is counted
+      if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
   wait_vm<0>();
-  if (tid == 0) {
-    if (atomicAdd(&g_exited, 1u) == (unsigned)G - 1) {  // last one out resets the counters
-      __hip_atomic_store(&g_arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
 }
 
 }  // namespace
 
 // (external linkage: the host takes its address for hipFuncSetAttribute)
 template <int MCAP, int NS>
-__global__ __launch_bounds__(kThreads) void gemv_stream_kernel(const void *entries, int n_entries, int *status) {
+__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int *status) {
   gemv_stream_body<MCAP, NS>(reinterpret_cast<const Entry *>(entries), n_entries, status);
 }
 
@@ -285,7 +421,7 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   for (int64_t i = 0; i < count && supported; ++i) {
     const gq_gemv_desc &d = host[i];
     if (d.m_rows > max_m) max_m = d.m_rows;
-    supported = d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.m_rows >= 1 && d.m_rows <= 8 &&
+    supported = d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.m_rows >= 1 && d.m_rows <= 4 &&
                 d.n_out >= 1 && ((uintptr_t)d.x % 16) == 0 && ((uintptr_t)d.packed % 16) == 0 &&
                 ((uintptr_t)d.scale % 16) == 0 && ((uintptr_t)d.bias % 16) == 0;
   }
@@ -310,11 +446,11 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     if (e != hipSuccess || n <= 0) return fail((int)e, "cannot query the compute unit count");
     cu_count[dev] = n;
   }
-  const int grid = cu_count[dev];  // one workgroup per compute unit: all of them are resident together
-  const void *entries = device;
+  const int grid = cu_count[dev] < kMaxGroups ? cu_count[dev] : kMaxGroups;  // one workgroup per compute unit, all resident together
 #define GQ_STREAM(MCAP, NS)                                                                                   \
   do {                                                                                                        \
-    constexpr int lds_bytes = kWaves * (NS * kItemBytes + MCAP * 1024);                                       \
+    constexpr int lds_bytes =                                                                                 \
+        kWaves * (NS * kItemBytes + MCAP * 1024) + kMaxEntries * 64 + kWaves * kPassRows * 4 * MCAP * 16 + 64;  \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
     auto kern = gemv_stream_kernel<MCAP, NS>;                                                                 \
     static bool configured = false;                                                                           \
@@ -324,10 +460,12 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
       if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
       configured = true;                                                                                      \
     }                                                                                                         \
-    kern<<<dim3(grid), dim3(kThreads), lds_bytes, stream>>>(entries, (int)count, status);                     \
+    for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
+      const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
+      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status);                     \
+    }                                                                                                         \
   } while (0)
-  if (max_m <= 4) GQ_STREAM(4, 3);
-  else GQ_STREAM(8, 2);
+  GQ_STREAM(4, 3);
 #undef GQ_STREAM
   return check_launch("gemv_stream_kernel");
 }
