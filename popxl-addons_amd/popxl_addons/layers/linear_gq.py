@@ -148,6 +148,40 @@ class LinearGQ:
 
     __call__ = build
 
+    # ------------------------------------------------------------------------------- fusion
+
+    @classmethod
+    def fuse(cls, layers):
+        """One layer computing the concatenated outputs of `layers` (e.g. the Q, K and V projections
+        of a decoder block, which read the same activations): y = cat([l(x) for l in layers], -1) in
+        a single kernel pass over x.  Needs groups along the input features (dim=0), where the
+        variables of the layers stack along their first axis; all layers must agree in
+        group_size, bias and input width.  The new layer owns copies of the variables.
+        """
+        import torch
+
+        layers = list(layers)
+        if not layers:
+            raise ValueError("LinearGQ.fuse: no layers")
+        first = layers[0]
+        for layer in layers:
+            if layer.variables is None:
+                raise ValueError("LinearGQ.fuse: every layer needs its variables (build it or call init_variables)")
+            if layer.dim != 0:
+                raise NotImplementedError("LinearGQ.fuse: only dim=0 layers stack along the output features")
+            if layer.group_size != first.group_size or layer.bias != first.bias:
+                raise ValueError("LinearGQ.fuse: layers differ in group_size or bias")
+            if layer.variables.weight_compressed.shape[1:] != first.variables.weight_compressed.shape[1:]:
+                raise ValueError("LinearGQ.fuse: layers differ in input features")
+        fused = cls(sum(l.out_features for l in layers), bias=first.bias, group_size=first.group_size, dim=0)
+        names = ["weight_compressed", "weight_decompression_scale", "weight_decompression_bias"]
+        if first.bias:
+            names.append("bias")
+        fused.variables = NamedTensors(
+            **{n: Variable(n, torch.cat([l.variables[n].data for l in layers], dim=0).contiguous()) for n in names}
+        )
+        return fused
+
     # ------------------------------------------------------------------------- weight mapping
 
     @staticmethod

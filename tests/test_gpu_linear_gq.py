@@ -98,3 +98,60 @@ def test_device_compress_config2_and_nonfinite(hip, device, oracle):
     w[7, 9] = np.nan
     with pytest.raises(ValueError):
         group_quantize_compress(to_dev(w, device), 64)
+
+
+@pytest.mark.parametrize("dim", [0, -1])
+def test_checkpoint_round_trip_on_device(hip, device, dim, tmp_path):
+    """A layer written to disk (one .npz per variable) and read into a fresh layer gives the same bits."""
+    from popxl_addons import checkpoint
+
+    in_features, out_features, group_size = 256, 512, 64
+    torch.manual_seed(1)
+    nn_layer = torch.nn.Linear(in_features, out_features)
+    layer = LinearGQ(out_features, bias=True, group_size=group_size, dim=dim)
+    variables = layer.init_variables(in_features, torch.float16, device)
+    layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=dim))
+    x = torch.randn((6, in_features), device=device, dtype=torch.float16)
+    y = layer(x)
+
+    checkpoint.save_layer(str(tmp_path), "block.proj", layer)
+    restored = LinearGQ(out_features, bias=True, group_size=group_size, dim=dim)
+    restored.init_variables(in_features, torch.float16, device)
+    checkpoint.load_layer(str(tmp_path), "block.proj", restored)
+    assert_bits_equal(restored(x).cpu().numpy(), y.cpu().numpy())
+
+
+@pytest.mark.parametrize("batch", [1, 4, 40])
+def test_fused_qkv_equals_separate_projections(hip, device, batch):
+    """Q, K and V read the same activations: stacking their variables gives one kernel pass whose
+    output is the concatenation of the three, bit for bit (every output row is computed from its
+    own weight row alone)."""
+    in_features, out_features, group_size = 512, 384, 64
+    torch.manual_seed(2)
+    layers = []
+    for _ in range(3):
+        nn_layer = torch.nn.Linear(in_features, out_features)
+        layer = LinearGQ(out_features, bias=True, group_size=group_size, dim=0)
+        variables = layer.init_variables(in_features, torch.float16, device)
+        layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=0))
+        layers.append(layer)
+    fused = LinearGQ.fuse(layers)
+    assert fused.out_features == 3 * out_features
+    x = torch.randn((batch, in_features), device=device, dtype=torch.float16)
+    want = torch.cat([layer(x) for layer in layers], dim=-1)
+    assert_bits_equal(fused(x).cpu().numpy(), want.cpu().numpy())
+
+
+def test_fuse_rejects_mismatched_layers(hip, device):
+    a = LinearGQ(64, bias=True, group_size=16, dim=0)
+    a.init_variables(64, torch.float16, device)
+    b = LinearGQ(64, bias=True, group_size=32, dim=0)
+    b.init_variables(64, torch.float16, device)
+    with pytest.raises(ValueError):
+        LinearGQ.fuse([a, b])
+    c = LinearGQ(64, bias=True, group_size=16, dim=-1)
+    c.init_variables(64, torch.float16, device)
+    with pytest.raises(NotImplementedError):
+        LinearGQ.fuse([a, c])
+    with pytest.raises(ValueError):
+        LinearGQ.fuse([])
