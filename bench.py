@@ -192,17 +192,41 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     ms = time_launches(lambda _: graph.replay(), passes, warmup)
     results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                                    "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS}
-    # (2) the whole stack as one gq_gemv_sequence_f16 call.  Dependencies as in a decoder layer: the
-    # q projection waits for the previous layer, k and v share its input, then o, up and down wait
-    # for their predecessor (4 device-wide synchronisations per layer).
-    seq = hip.GemvSequence(device)
-    for i, (n_out, k_in, p, s, b) in enumerate(mats):
-        seq.add(xs[k_in], p, s, b, ys[i % 6], None, wait_previous=(i % 6) in (0, 3, 4, 5) and i > 0)
-    ms = time_launches(lambda _: seq.run(), passes, warmup)
-    torch.cuda.synchronize()
-    results["sequence"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
-                           "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
-                           "syncs_per_pass": sum(1 for i in range(len(mats)) if (i % 6) in (0, 3, 4, 5) and i > 0)}
+    # (2) the whole stack as one gq_gemv_sequence_f16 call, with the dependencies of a decoder layer
+    # declared per entry.  Roles per layer, in `mats` order: q k v o up down.
+    #   sequential block   q waits for the previous layer, k and v share its input, then o, up and
+    #                      down each wait for their predecessor (4 device-wide waits per layer)
+    #   parallel block     attention and feed-forward read the same layer input (the 6B model of
+    #                      these shapes is built that way): order q k v up o down; q waits for the
+    #                      previous layer, o for v (up streams meanwhile), down for up
+    #   no waits           no dependencies: the streaming rate of the kernel alone, not a decoder
+    def sequential(seq):
+        for i, (n_out, k_in, p, s, b) in enumerate(mats):
+            seq.add(xs[k_in], p, s, b, ys[i % 6], None, wait_previous=(i % 6) in (0, 3, 4, 5))
+
+    def parallel(seq):
+        last = None
+        for layer in range(n_layers):
+            idx = {}
+            for role in (0, 1, 2, 4, 3, 5):
+                n_out, k_in, p, s, b = mats[layer * 6 + role]
+                wait_for = {0: last, 3: idx.get(2), 5: idx.get(4)}.get(role)
+                idx[role] = seq.add(xs[k_in], p, s, b, ys[role], None, wait_for=wait_for)
+            last = idx[5]
+
+    def free(seq):
+        for i, (n_out, k_in, p, s, b) in enumerate(mats):
+            seq.add(xs[k_in], p, s, b, ys[i % 6], None)
+
+    for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
+                       ("sequence_no_waits", free)):
+        seq = hip.GemvSequence(device)
+        fill(seq)
+        ms = time_launches(lambda _: seq.run(), passes, warmup)
+        torch.cuda.synchronize()
+        results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                         "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
+                         "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0)}
     return results
 
 
@@ -287,7 +311,7 @@ def main():
         for m in (1, 4):
             r = bench_stack(hip, device, m, passes=20, warmup=3)
             extra["stack"].append(r)
-            for mode in ("per_launch_graph", "sequence"):
+            for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block", "sequence_no_waits"):
                 log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
                     f"({r[mode]['hbm_frac']:.1%})")
             torch.cuda.empty_cache()

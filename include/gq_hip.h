@@ -117,12 +117,14 @@ int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, con
  * A sequence of decode GEMVs (a layer stack) as one call.  No counterpart in the reference, where
  * a model is a chain of LinearGQ.build calls (popxl_addons/layers/linear_gq.py:99-109) compiled
  * into one static device program; this entry point is the analogue for a chain of gq_gemv_f16
- * calls: entry i computes exactly what gq_gemv_f16 would, entries run in order, and an entry with
- * wait_previous != 0 starts only after every earlier entry has completed (set it when x or
- * out_bias of the entry is produced by an earlier one).  Entries without the flag may overlap
- * earlier ones.
+ * calls: entry i computes exactly what gq_gemv_f16 would.  Dependencies between entries are
+ * declared, not implied: entry i starts only after the first wait_entries[i] entries of the
+ * sequence have completed (0 <= wait_entries <= i; 0 = no dependency, i = every earlier entry).
+ * Set it past the entry that produces x or out_bias of entry i.  Entries may otherwise overlap
+ * and complete in any order: an entry that overwrites memory which an earlier entry reads or
+ * writes must wait for that entry as well.
  *
- * For group_size 64, k_in % 512 == 0, m_rows <= 8 and 16-byte aligned pointers the whole sequence
+ * For group_size 64, k_in % 512 == 0, m_rows <= 4 and 16-byte aligned pointers the whole sequence
  * runs as one persistent kernel (one workgroup per compute unit) that streams the packed weights
  * without a gap between entries; any other sequence runs as one launch per entry.
  *
@@ -141,7 +143,7 @@ typedef struct gq_gemv_desc {
   const uint16_t *out_bias; /* [n_out] binary16 or NULL */
   uint16_t *y;              /* [m_rows, n_out] binary16 */
   int32_t m_rows, n_out, k_in, group_size;
-  int32_t wait_previous;
+  int32_t wait_entries;     /* entries [0, wait_entries) complete before this one starts */
   int32_t reserved;         /* 0 */
 } gq_gemv_desc;
 

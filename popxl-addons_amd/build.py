@@ -30,6 +30,9 @@ FLAGS = [
 
 # kernels whose result must be bit-exact: no fused fp16 multiply-add may appear in their ISA
 NO_FMA_SOURCES = {"gq_decompress.hip": r"v_(pk_)?(fma|mad|fmac)_f16|v_fma_mix"}
+# kernels that count their outstanding vector-memory operations by hand (s_waitcnt vmcnt(N) with
+# direct-to-LDS loads): a register spill would add scratch accesses to that count
+NO_SCRATCH_SOURCES = ["gq_gemv_stream.hip", "gq_gemm.hip"]
 
 
 def _run(cmd):
@@ -57,6 +60,12 @@ def check_isa():
             raise RuntimeError(f"{src}: fused fp16 multiply-add in ISA ({sorted(set(map(str, hits)))})")
         if "v_pk_mul_f16" not in text or "v_pk_add_f16" not in text:
             raise RuntimeError(f"{src}: expected v_pk_mul_f16 and v_pk_add_f16 in ISA")
+    for src in NO_SCRATCH_SOURCES:
+        asm = os.path.join(OBJ_DIR, src.replace(".hip", ".s"))
+        _run([HIPCC, *FLAGS, "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", asm])
+        text = open(asm).read()
+        if re.search(r"^\s*scratch_(load|store)", text, re.M):
+            raise RuntimeError(f"{src}: registers spill to scratch memory")
 
 
 def build(check=True, jobs=None):

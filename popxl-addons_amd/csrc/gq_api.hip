@@ -160,6 +160,9 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
     if (d.m_rows > 16)
       return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld has m_rows=%d > 16", (long long)i,
                       d.m_rows);
+    if (d.wait_entries < 0 || d.wait_entries > i)
+      return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: entry %lld has wait_entries=%d outside [0, %lld]",
+                      (long long)i, d.wait_entries, (long long)i);
   }
   return gq::launch_gemv_sequence(descs, descs_device, count, status, (hipStream_t)stream);
 }

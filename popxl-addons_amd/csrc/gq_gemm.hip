@@ -546,7 +546,7 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
       case 1: return GQ_PIPE2(1, 4, 8, 1, 3, 1);  // 256 x 128, 4 waves of 256 x 32
       case 2: return GQ_PIPE2(1, 4, 4, 1, 3, 2);  // 128 x 128, 4 waves of 128 x 32, two workgroups per CU
       case 3: return GQ_PIPE2(1, 4, 4, 2, 3, 2);  // 128 x 256, 4 waves of 128 x 64, two workgroups per CU
-      default: return GQ_PIPE2(2, 2, 4, 2, 3, 2);  // 256 x 128, 4 waves of 128 x 64
+      default: return GQ_PIPE2(2, 2, 4, 2, 3, 1);  // 256 x 128, 4 waves of 128 x 64
     }
   }
 #undef GQ_PIPE2

@@ -5,16 +5,26 @@
 // whole list of entries.  Packed weights, scales and biases never depend on earlier results, so
 // every wave streams them through a private LDS ring with direct-to-LDS loads that run several
 // work items ahead -- across entry boundaries -- while only the small activation vector x waits
-// for the entries it depends on (a device-wide counter, bounded spin).
+// for the entries it depends on (per-workgroup progress words, bounded spin).
 //
-// Work decomposition of one entry (n_out x k_in, k_in % 512 == 0, group 64, m_rows <= MCAP):
-//   row block  = 16 weight rows; workgroup b of G owns row blocks b, b + G, ... in passes of 4
+// Work decomposition of one entry (n_out x k_in, k_in % 512 == 0, group 64, m_rows <= 4):
+//   row block  = 16 weight rows; workgroup b of G owns row blocks b, b + G, ... in passes of 4 (2 when MC = 4)
 //   phase      = 4096 contraction indices; wave w owns chunk 8 p + w (512 indices) of phase p
 //   work item  = (row block, chunk): 4 KiB of packed words + 2 x 256 B of scale / bias
-// A wave keeps the permuted x fragments of its chunk in registers and re-uses them for the row
-// blocks of the pass; the 16 x 16 partial sums of the 8 waves meet in LDS at the end of a pass.
-// The arithmetic is that of gemv_mfma_kernel (v_mfma_f32_16x16x32_f16, codes expanded in pair
-// order, x permuted to match).
+//
+// Arithmetic.  Once the weights stream without gaps the loop is bound by instruction issue, not by
+// HBM, so the expansion of the codes is kept to 5 VALU instructions per 8 weights: a code is only
+// or-ed into the mantissa of 64.0 or 1024.0 (exact: 64 + c or 1024 + c) and goes to the MFMA as
+// it is.  Scale and bias are applied to SUMS instead of weights:
+//   y[n] = sum_g scale[n][g] * ( sum_{k in g} (off_k + c[n][k]) x[k]  -  sum_{k in g} off_k x[k] )
+//        + sum_g bias[n][g]  *   sum_{k in g} x[k]
+// v_mfma_f32_16x16x32_f16 computes D[i][n] += sum_k A[i][k] B[k][n].  B holds the raw codes of 16
+// weight rows n; A holds x, its sixteen rows i used as (group, batch row) combinations: row i of A
+// is x[m(i)] on the contraction indices of group g(i) and zero elsewhere.  One accumulator thus
+// separates the groups of a whole item (MC = 2: 8 groups x 2 batch rows) or of half an item
+// (MC = 4: 4 groups x 4 batch rows), and a lane finds in its 4 accumulator registers group sums of
+// ITS weight row.  The per-group corrections sum off_k x[k] and sum x[k] are computed once per x
+// chunk (v_dot2_f32_f16, fp32 accumulation).
 #include "gq_common.h"
 #include "gq_gemv_dequant.h"
 
@@ -24,8 +34,10 @@ namespace {
 constexpr int kWaves = 8;                         // compute waves
 constexpr int kThreadsAll = (kWaves + 2) * 64;    // + reducer + poller
 constexpr int kItemBytes = 4096 + 512;  // packed words, 16 rows x 16 B of scale, 16 rows x 16 B of bias
-constexpr int kItemOps = 5;             // direct-to-LDS loads per item: 4 packed + 1 scale/bias
-constexpr int kPassRows = 4;            // row blocks per pass (accumulators held by a wave)
+constexpr int kItemOps = 6;             // direct-to-LDS loads per item: 4 packed + scale + bias
+// row blocks per pass (a wave holds their running sums in registers and re-uses the x operands
+// for them); the variant for 4 batch rows has fewer registers to spare
+constexpr int pass_rows(int mc) { return mc == 2 ? 4 : 2; }
 constexpr unsigned kSpinLimit = 1u << 18;
 
 // Progress of the running sequence on this device.  Every workgroup publishes the number of
@@ -43,7 +55,7 @@ struct Entry {  // = gq_gemv_desc
   const half_t *bias;
   const half_t *out_bias;
   half_t *y;
-  int32_t m_rows, n_out, k_in, group_size, wait_previous, reserved;
+  int32_t m_rows, n_out, k_in, group_size, wait_entries, reserved;
 };
 static_assert(sizeof(Entry) == sizeof(gq_gemv_desc), "descriptor layout");
 
@@ -54,18 +66,19 @@ __device__ __forceinline__ void wait_vm() {
 
 // position of a wave in the list of its work items
 struct Cursor {
-  int d, pass, phase, j;  // entry, pass of 4 row blocks, phase of 4096 indices, row block in pass
+  int d, pass, phase, j;  // entry, pass of row blocks, phase of 4096 indices, row block in pass
 };
 
 // what the kernel needs of an entry, kept in LDS: descriptor reads from global memory in the
 // work loop cost microseconds each
 struct CachedEntry {
-  const uint4_t *packed;
-  const half_t *scale, *bias, *x, *out_bias;
+  const char *packed, *scale, *bias;
+  const half_t *x, *out_bias;
   half_t *y;
   int n_out, k_in;
-  short m_rows, wait_previous;
-  int nrb;  // row blocks owned by this workgroup
+  short m_rows, wait;  // wait: entries of this launch that must be complete before this one starts
+  short nrb;           // row blocks owned by this workgroup
+  short publish;       // somebody waits for exactly this entry and its predecessors: report its completion
 };
 static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
 constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
@@ -86,60 +99,94 @@ __device__ __forceinline__ unsigned lds_load(const unsigned *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// MCAP: largest batch (the x stage of a wave holds MCAP KiB); NS: depth of the weight ring.
-// (A __device__ function: a __global__ template is also instantiated for the host, where the
-// target builtins and inline assembly do not exist.)
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const char *uni_ptr(const void *p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  return (const char *)(uintptr_t)(((uint64_t)(uint32_t)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v));
+}
+__device__ __forceinline__ float lane_read(float v, int src_lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v)));
+}
+
+// 8 codes of `w` as fp16 (64 + c) or (1024 + c), order (0,4,1,5,2,6,3,7): 5 VALU instructions.
+// Codes 0,2 (and 4,6) sit at bits 7:4 of a byte and land in the mantissa of 64.0 (ulp 1/16 x 16);
+// codes 1,3 (5,7) sit at bits 3:0 and land in the mantissa of 1024.0 (ulp 1).
+__device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint32_t mask_hi, uint32_t magic_lo,
+                                             uint32_t magic_hi) {
+  const uint32_t hi = w >> 8;
+  uint4_t v;
+  v.x = and_or(hi, mask_hi, magic_hi);  // codes 0, 4: 64 + c
+  v.y = and_or(hi, mask_lo, magic_lo);  // codes 1, 5: 1024 + c
+  v.z = and_or(w, mask_hi, magic_hi);   // codes 2, 6: 64 + c
+  v.w = and_or(w, mask_lo, magic_lo);   // codes 3, 7: 1024 + c
+  return __builtin_bit_cast(half8_t, v);
+}
+
+// MC: batch rows a launch can hold (2 or 4; the x stage of a wave holds MC KiB); NS: depth of the
+// weight ring.  (A __device__ function: a __global__ template is also instantiated for the host,
+// where the target builtins and inline assembly do not exist.)
 //
 // Waves 0..7 compute; they never meet at a workgroup barrier.  After the last chunk of a pass a
 // wave drops its 16 x m partial sums into its mailbox and goes on with the next pass or entry.
-// Wave 8, the reducer, adds the eight mailboxes in a fixed order, stores y and counts the
-// workgroup as arrived for the entry.  Wave 9, the poller, watches the device-wide arrival count
-// and publishes in LDS how many entries are complete; a compute wave that needs an earlier result
-// waits for that number only.
+// Wave 8, the reducer, adds the eight mailboxes in a fixed order, stores y and, for entries that
+// somebody waits for, publishes the workgroup's progress.  Wave 9, the poller, watches the
+// progress words of all workgroups and publishes in LDS how many entries are complete everywhere;
+// a compute wave that needs an earlier result waits for that number only.
 //
 // Visibility of results between compute units needs no cache flush: y is written with device-scope
 // stores (sc1, write-through to the coherent level), the reducer waits for its stores before it
-// counts, and x is read with device-coherent loads.
-template <int MCAP, int NS>
-__device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries,
+// publishes, and x is read with device-coherent loads.
+template <int MC, int NS>
+__device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries, int first_entry,
                                                  int *__restrict__ status) {
+  static_assert(MC == 2 || MC == 4, "batch capacity");
+  constexpr int PR = pass_rows(MC);
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int kWaveBytes = NS * kItemBytes + MCAP * 1024;
-  constexpr int kMailBytes = kPassRows * 4 * MCAP * 16;  // per wave: [row block][kc][m] float4
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int kWaveBytes = NS * kItemBytes + MC * 1024;
+  constexpr int kMailFloats = PR * MC * 16;  // per wave: [row block][m][n]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
   const int r = lane & 15, kc = lane >> 4;
   const int G = gridDim.x, b = blockIdx.x;
   CachedEntry *cache = reinterpret_cast<CachedEntry *>(lds + kWaves * kWaveBytes);
-  char *mail = lds + kWaves * kWaveBytes + kMaxEntries * 64;
-  Control *ctl = reinterpret_cast<Control *>(mail + kWaves * kMailBytes);
+  float *mail = reinterpret_cast<float *>(lds + kWaves * kWaveBytes + kMaxEntries * 64);
+  Control *ctl = reinterpret_cast<Control *>(mail + kWaves * kMailFloats);
+  // MC == 4 only: per wave, the group sums of the current x chunk, [half][kc][corr e0..3, xsum e0..3]
+  // (registers are short in that variant)
+  float *table = reinterpret_cast<float *>(ctl) + 16 + wave * 64;
 
   for (int i = tid; i < n_entries; i += kThreadsAll) {
     const Entry e = entries[i];
     CachedEntry c;
-    c.packed = e.packed;
-    c.scale = e.scale;
-    c.bias = e.bias;
+    c.packed = reinterpret_cast<const char *>(e.packed);
+    c.scale = reinterpret_cast<const char *>(e.scale);
+    c.bias = reinterpret_cast<const char *>(e.bias);
     c.x = e.x;
     c.out_bias = e.out_bias;
     c.y = e.y;
     c.n_out = e.n_out;
     c.k_in = e.k_in;
     c.m_rows = (short)e.m_rows;
-    c.wait_previous = (short)(e.wait_previous != 0);
+    c.wait = (short)max(0, e.wait_entries - first_entry);  // earlier launches are complete
     const int rb = (e.n_out + 15) >> 4;
-    c.nrb = rb > b ? (rb - b + G - 1) / G : 0;
+    c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
+    c.publish = 0;
     cache[i] = c;
   }
   if (tid == 0) *ctl = Control{0u, 0u, 0u, 0u};
-  __syncthreads();  // the only workgroup barrier
-
-  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  __syncthreads();
+  // completion is reported only where an entry waits for it (a report costs the reducer a round
+  // trip to memory)
+  for (int i = tid; i < n_entries; i += kThreadsAll) {
+    const int w = cache[i].wait;
+    if (w > 0) cache[w - 1].publish = 1;
+  }
+  __syncthreads();
 
   // ============================================================================ poller
   if (wave == kWaves + 1) {
-    int last_waited = 0;
-    for (int d = 1; d < n_entries; ++d)
-      if (cache[d].wait_previous) last_waited = d;
+    int last_waited = 0;  // the largest count anybody waits for
+    for (int d = 1; d < n_entries; ++d) last_waited = max(last_waited, (int)cache[d].wait);
     // one 16-byte device-coherent load per lane covers 256 workgroups; the minimum over all of them
     // is the number of entries complete everywhere
     unsigned ready = 0, spins = 0;
@@ -181,44 +228,39 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), n_out = uni(cache[d].n_out);
       half_t *y = cache[d].y;
       const half_t *out_bias = cache[d].out_bias;
-      for (int pass = 0; pass * kPassRows < nrb; ++pass, ++q) {
-        const int nj = min(kPassRows, nrb - pass * kPassRows);
+      for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
+        const int nj = min(PR, nrb - pass * PR);
         while (lds_load(&ctl->deposited) < (q + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
-        // lane -> (row block j, kc, m): 16 lanes per row block when MCAP == 4
-        for (int t = lane; t < nj * 4 * MCAP; t += 64) {
-          const int m = t % MCAP, kq = (t / MCAP) & 3, j = t / (4 * MCAP);
-          float4_t sum = {0.f, 0.f, 0.f, 0.f};
+        // one sum per (row block j, batch row m, output n): consecutive lanes, consecutive n
+        for (int t = lane; t < nj * MC * 16; t += 64) {
+          const int n16 = t & 15, m = (t >> 4) % MC, j = t / (16 * MC);
+          float sum = 0.f;
 #pragma unroll
-          for (int w = 0; w < kWaves; ++w) sum += *reinterpret_cast<const float4_t *>(mail + w * kMailBytes + t * 16);
-          if (m < m_rows) {
-            const int n0 = (b + (pass * kPassRows + j) * G) * 16 + 4 * kq;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int n = n0 + i;
-              if (n < n_out) {
-                float v = sum[i];
-                if (out_bias) v += (float)out_bias[n];
-                const half_t hv = (half_t)v;
-                // device-scope store: written through to where every compute unit reads it
-                __hip_atomic_store(reinterpret_cast<unsigned short *>(y) + (int64_t)m * n_out + n,
-                                   __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-              }
-            }
+          for (int w = 0; w < kWaves; ++w) sum += mail[w * kMailFloats + t];
+          const int n = (b + (pass * PR + j) * G) * 16 + n16;
+          if (m < m_rows && n < n_out) {
+            if (out_bias) sum += (float)out_bias[n];
+            const half_t hv = (half_t)sum;
+            // device-scope store: written through to where every compute unit reads it
+            __hip_atomic_store(reinterpret_cast<unsigned short *>(y) + (int64_t)m * n_out + n,
+                               __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
         // the mailboxes have been read (the sums above depend on them): free them
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) __hip_atomic_store(&ctl->consumed, q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
-      wait_vm<0>();  // every lane's stores of this entry are complete ...
-      if (lane == 0)   // ... then publish
-        __hip_atomic_store(&g_progress[b], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (uni(cache[d].publish)) {
+        wait_vm<0>();  // every lane's stores of this and of all earlier entries are complete ...
+        if (lane == 0)   // ... then publish
+          __hip_atomic_store(&g_progress[b], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     // the last workgroup out clears the progress words: by then every poller has seen all it needs
     wait_vm<0>();  // this workgroup's last progress word is in memory before it counts itself out
     unsigned last = 0;
     if (lane == 0) last = atomicAdd(&g_exited, 1u) == (unsigned)G - 1;
-    if (__builtin_amdgcn_readfirstlane((int)last)) {
+    if (uni((int)last)) {
       wait_vm<0>();
       for (int i = lane; i < G; i += 64) __hip_atomic_store(&g_progress[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -230,15 +272,9 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   char *ring = lds + wave * kWaveBytes;
   char *xstage = ring + NS * kItemBytes;
   const uint32_t ring_rd = (uint32_t)(uintptr_t)ring, x_rd = (uint32_t)(uintptr_t)xstage;
-  const uint32_t half_sel = (kc & 2) ? 0x07060706u : 0x05040504u;  // lane's group within a slot: kc / 2
 
-  // The producer walks the same item list as the consumer, NS items ahead.  Its entry is held in
-  // scalar registers (values read from LDS are made wave-uniform explicitly), so that advancing
-  // the cursor is a handful of scalar instructions.
-  auto uni_ptr = [&](const void *p) {
-    const uint64_t v = (uint64_t)(uintptr_t)p;
-    return (const char *)(uintptr_t)(((uint64_t)(uint32_t)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v));
-  };
+  // ---- the producer walks the same item list as the consumer, NS items ahead.  Everything it
+  // needs is wave-uniform (scalar registers): advancing the cursor costs no vector instruction.
   struct ProducerEntry {
     const char *packed, *scale, *bias;
     int n_out, k_in, nrb, phases;
@@ -257,14 +293,14 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   // chunks past k_in are skipped)
   auto valid = [&](const Cursor &c) {
     if (c.d >= n_entries) return true;  // the end is a valid resting place
-    return c.pass * kPassRows + c.j < pe.nrb && (c.phase * kWaves + wave) * 512 < pe.k_in;
+    return c.pass * PR + c.j < pe.nrb && (c.phase * kWaves + wave) * 512 < pe.k_in;
   };
   auto step = [&](Cursor &c) {
-    if (++c.j < kPassRows && c.pass * kPassRows + c.j < pe.nrb) return;
+    if (++c.j < PR && c.pass * PR + c.j < pe.nrb) return;
     c.j = 0;
     if (++c.phase < pe.phases) return;
     c.phase = 0;
-    if (++c.pass * kPassRows < pe.nrb) return;
+    if (++c.pass * PR < pe.nrb) return;
     c.pass = 0;
     ++c.d;
     load_producer_entry(c.d);
@@ -273,20 +309,25 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     do step(c);
     while (c.d < n_entries && !valid(c));
   };
-  // direct-to-LDS loads of the item at cursor c into ring slot `slot`
+  // direct-to-LDS loads of the item at cursor c into ring slot `slot`: scalar base of the row
+  // block's chunk + one 32-bit offset per lane
   auto issue_item = [&](const Cursor &c, int slot) {
-    const int rb = b + (c.pass * kPassRows + c.j) * G;
-    const int row = min(rb * 16 + r, pe.n_out - 1);
+    const int rb = b + (c.pass * PR + c.j) * G;
     const int chunk = c.phase * kWaves + wave;
+    const int row = min(r, pe.n_out - 1 - rb * 16);  // rows past n_out re-read the last one
     char *dst = ring + slot * kItemBytes;
-    const uint4_t *src = reinterpret_cast<const uint4_t *>(pe.packed) + (int64_t)row * (pe.k_in >> 5) + chunk * 16 + kc;
+    const char *src = pe.packed + (int64_t)rb * 16 * (pe.k_in >> 1) + chunk * 256;
+    const uint32_t off = (uint32_t)row * (uint32_t)(pe.k_in >> 1) + (uint32_t)kc * 16u;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) __builtin_amdgcn_global_load_lds(src + s * 4, dst + s * 1024, 16, 0, 0);
-    // lanes kc == 0 fetch the 8 scales of their row's chunk, lanes kc == 1 the 8 biases
-    if (kc < 2) {
-      const half_t *sb = reinterpret_cast<const half_t *>(kc == 0 ? pe.scale : pe.bias) + (int64_t)row * (pe.k_in >> 6) + chunk * 8;
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(sb), dst + 4096, 16, 0, 0);
-    }
+    for (int s = 0; s < 4; ++s)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(src + off + s * 64), dst + s * 1024, 16, 0, 0);
+    // lanes 0..15 fetch the 8 scales of their row's chunk, lanes 16..31 the 8 biases
+    const uint32_t off2 = (uint32_t)row * (uint32_t)(pe.k_in >> 5);
+    const int64_t base2 = (int64_t)rb * 16 * (pe.k_in >> 5) + chunk * 16;
+    if (kc == 0)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.scale + base2 + off2), dst + 4096, 16, 0, 0);
+    if (kc == 1)
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.bias + base2 + off2), dst + 4096, 16, 0, 0);
   };
 
   Cursor prod = {0, 0, 0, 0};  // the producer's position: first item of this wave
@@ -301,63 +342,131 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   int slot = 0;    // ring slot of the consumer's item
   unsigned q = 0;  // passes finished so far (same count in every wave)
 
-  half8_t xp[4][4];
-  const half_t *x_loaded = nullptr;  // x fragments in registers belong to (x_loaded, chunk x_chunk)
+  // ---- lane roles
+  // B operand / loader: weight row r, 16-byte piece kc of every 64-byte stretch.
+  // A operand: combination i = r of (group, batch row); contraction slice kc.
+  // D: column n = r (weight row), rows 4 kc + e = combinations.
+  //   MC == 2: i = 2 g + m, g = 0..7: one accumulator per item; a lane's rows are groups 2kc, 2kc+1
+  //   MC == 4: i = 4 g + m, g = 0..3: accumulator A for groups 0..3 (loads 0, 1), B for 4..7
+  const int a_g = MC == 2 ? (r >> 1) : (r >> 2);  // group of this lane's A row (within its half for MC 4)
+  const int a_m = MC == 2 ? (r & 1) : (r & 3);
+  const int a_load = a_g >> 1;                     // the 16-byte load (128 indices) holding that group
+  const bool a_match = (kc >> 1) == (a_g & 1);     // ... and whether this lane's slice is in the group
+  const uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u, kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
+  const half2_t kOnes = {(half_t)1.0f, (half_t)1.0f};
+  const half2_t kOffsets = {(half_t)64.0f, (half_t)1024.0f};  // even index of a word: 64 + c, odd: 1024 + c
+
+  half8_t xa[4][4];                  // A operands of the 16 MFMA steps of an item
+  float corr[4] = {0.f, 0.f, 0.f, 0.f};  // MC 2: sum of off_k x[k] over the group of accumulator row e
+  float xsum[4] = {0.f, 0.f, 0.f, 0.f};  // MC 2: sum of x[k] over that group
+  const uint32_t table_rd = (uint32_t)(uintptr_t)table + kc * 32;
+#pragma unroll
+  for (int L = 0; L < 4; ++L)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xa[L][j] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  if (MC == 4 && r == 0) {
+    // the table must hold numbers before the first x chunk arrives (0 * NaN would poison a sum)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) table[(h * 4 + kc) * 8 + e] = 0.f;
+  }
+  const half_t *x_loaded = nullptr;  // the operands in registers belong to (x_loaded, chunk x_chunk)
   int x_chunk = -1, x_k = 0, x_m = 0;
+  unsigned known_ready = 0;  // entries this wave has seen complete on the whole device
 
   for (int d = 0; d < n_entries; ++d) {
     const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), k_in = uni(cache[d].k_in);
     const half_t *x = reinterpret_cast<const half_t *>(uni_ptr(cache[d].x));
     const int phases = (k_in + 4095) >> 12;
-    if (uni(cache[d].wait_previous) && d > 0) {
-      // every workgroup has finished every earlier entry (published by the poller)
-      while (lds_load(&ctl->ready) < (unsigned)d && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
+    const unsigned need = (unsigned)uni(cache[d].wait);
+    if (need > known_ready) {
+      // every workgroup has finished the first `need` entries (published by the poller)
+      while ((known_ready = lds_load(&ctl->ready)) < need && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
       x_loaded = nullptr;
     }
-    for (int pass = 0; pass * kPassRows < nrb; ++pass, ++q) {
-      const int nj = min(kPassRows, nrb - pass * kPassRows);
-      float4_t acc[kPassRows];
+    for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
+      const int nj = min(PR, nrb - pass * PR);
+      float4_t tot[PR];  // running sums: scale and bias applied, groups not yet added up
 #pragma unroll
-      for (int j = 0; j < kPassRows; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < PR; ++j) tot[j] = float4_t{0.f, 0.f, 0.f, 0.f};
       for (int phase = 0; phase < phases; ++phase) {
         const int chunk = phase * kWaves + wave;
         if (chunk * 512 >= k_in) continue;
-        // ---- x fragments of this chunk (kept when the previous entry used the same ones)
+        // ---- A operands and group sums of this chunk (kept when the previous entry used the same x)
         const bool reload_x = !(x_loaded == x && x_chunk == chunk && x_k == k_in && x_m == m_rows);
         if (reload_x) {
           for (int m = 0; m < m_rows; ++m)
             __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
                                              xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
           wait_vm<0>();  // x is the youngest load: everything in flight lands with it
-          uint4_t xq[4][4];
+          const bool active = a_match && a_m < m_rows;
+          constexpr int HALVES = MC == 2 ? 1 : 2;
+          float part_sum[HALVES], part_corr[HALVES];
 #pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4)
+          for (int h = 0; h < HALVES; ++h) {
+            // this lane's 32 indices of its group: 4 x 8 consecutive fp16 at (load, slice kc)
+            const int load = a_load + 2 * h;
+            uint4_t xq[4];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) xq[j4][s] = uint4_t{0u, 0u, 0u, 0u};
-          if (r < m_rows) {
+            for (int j = 0; j < 4; ++j)
+              asm volatile("ds_read_b128 %0, %1 offset:%2"
+                           : "=v"(xq[j])
+                           : "v"(x_rd + a_m * 1024 + (4 * load + kc) * 64), "n"(j * 16));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xq[0]), "+v"(xq[1]), "+v"(xq[2]), "+v"(xq[3]));
+            float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-            for (int j4 = 0; j4 < 4; ++j4)
+            for (int j = 0; j < 4; ++j) {
+              if (!active) xq[j] = uint4_t{0u, 0u, 0u, 0u};  // rows of x that were not loaded may hold anything
 #pragma unroll
-              for (int s = 0; s < 4; ++s)
-                asm volatile("ds_read_b128 %0, %1 offset:%2"
-                             : "=v"(xq[j4][s])
-                             : "v"(x_rd + r * 1024 + kc * 64), "n"((j4 * 16 + s) * 16));
-          }
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+              for (int t = 0; t < 4; ++t) {
+                s1 = __builtin_amdgcn_fdot2(as_half2(xq[j][t]), kOnes, s1, false);
+                s2 = __builtin_amdgcn_fdot2(as_half2(xq[j][t]), kOffsets, s2, false);
+              }
+              const half8_t p = permute_x(xq[j]);
+              if (MC == 2) {
 #pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4)
+                for (int L = 0; L < 4; ++L) xa[L][j] = a_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+              } else {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-              asm volatile("" : "+v"(xq[j4][s]));  // consumed after the wait
-              xp[j4][s] = permute_x(xq[j4][s]);
+                for (int L = 0; L < 2; ++L) xa[L + 2 * h][j] = a_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+              }
             }
+            // the other half of the group sits in the neighbouring slice
+            part_sum[h] = s1 + lane_read(s1, lane ^ 16);
+            part_corr[h] = s2 + lane_read(s2, lane ^ 16);
+          }
+          // accumulator row e of lane (n, kc) is combination 4 kc + e: fetch its sums from a lane
+          // that holds that A row and whose slice lies in the group
+#pragma unroll
+          for (int h = 0; h < HALVES; ++h) {
+            float4_t cs, xs;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int i = 4 * kc + e;
+              const int g = MC == 2 ? (i >> 1) : (i >> 2);
+              const int src = i + 32 * (g & 1);
+              xs[e] = lane_read(part_sum[h], src);
+              cs[e] = lane_read(part_corr[h], src);
+            }
+            if (MC == 2) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                xsum[e] = xs[e];
+                corr[e] = cs[e];
+              }
+            } else if (r == 0) {
+              *reinterpret_cast<float4_t *>(table + (h * 4 + kc) * 8) = cs;
+              *reinterpret_cast<float4_t *>(table + (h * 4 + kc) * 8 + 4) = xs;
+            }
+          }
           x_loaded = x;
           x_chunk = chunk;
           x_k = k_in;
           x_m = m_rows;
         }
 #pragma unroll
-        for (int j = 0; j < kPassRows; ++j) {
+        for (int j = 0; j < PR; ++j) {
           if (j >= nj) break;
           // ---- this item's loads are older than those of the n_ahead - 1 items issued after it
           if (!reload_x || j > 0) {
@@ -367,12 +476,24 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             else wait_vm<0>();
           }
           const uint32_t src = ring_rd + slot * kItemBytes;
-          uint4_t wq[4], sv, bv;
+          uint4_t wq[4];
+          uint32_t sA = 0, bA = 0, sB = 0, bB = 0;
 #pragma unroll
-          for (int s = 0; s < 4; ++s) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wq[s]) : "v"(src + lane * 16), "n"(s * 1024));
-          asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(sv) : "v"(src + r * 16));
-          asm volatile("ds_read_b128 %0, %1 offset:4352" : "=v"(bv) : "v"(src + r * 16));
-          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]), "+v"(sv), "+v"(bv));
+          for (int L = 0; L < 4; ++L) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(wq[L]) : "v"(src + lane * 16), "n"(L * 1024));
+          if (MC == 2) {
+            // (scale[2kc], scale[2kc+1]) of row r: the groups of this lane's accumulator rows
+            asm volatile("ds_read_b32 %0, %1 offset:4096" : "=v"(sA) : "v"(src + r * 16 + kc * 4));
+            asm volatile("ds_read_b32 %0, %1 offset:4352" : "=v"(bA) : "v"(src + r * 16 + kc * 4));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]), "+v"(sA), "+v"(bA));
+          } else {
+            // scale[kc] (half A) and scale[4 + kc] (half B) of row r
+            asm volatile("ds_read_u16 %0, %1 offset:4096" : "=v"(sA) : "v"(src + r * 16 + kc * 2));
+            asm volatile("ds_read_u16 %0, %1 offset:4104" : "=v"(sB) : "v"(src + r * 16 + kc * 2));
+            asm volatile("ds_read_u16 %0, %1 offset:4352" : "=v"(bA) : "v"(src + r * 16 + kc * 2));
+            asm volatile("ds_read_u16 %0, %1 offset:4360" : "=v"(bB) : "v"(src + r * 16 + kc * 2));
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]), "+v"(sA), "+v"(bA), "+v"(sB), "+v"(bB));
+          }
           // ---- the slot is free: fetch the item NS ahead into it
           --n_ahead;
           if (prod.d < n_entries) {
@@ -381,23 +502,69 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             next_item(prod);
           }
           slot = slot + 1 == NS ? 0 : slot + 1;
-          // ---- expand and multiply
+          // ---- multiply raw codes, then scale the group sums
+          if (MC == 2) {
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int j4 = 0; j4 < 4; ++j4) {
-            const half2_t s2 = as_half2(__builtin_amdgcn_perm(sv[j4], sv[j4], half_sel));
-            const half2_t b2 = as_half2(__builtin_amdgcn_perm(bv[j4], bv[j4], half_sel));
+            for (int L = 0; L < 4; ++L)
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
-              acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant_word(wq[j4][s], s2, b2), xp[j4][s], acc[j], 0, 0, 0);
+              for (int w = 0; w < 4; ++w)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[L][w], raw_codes(wq[L][w], kMaskLo, kMaskHi, kMagicLo, kMagicHi),
+                                                             acc, 0, 0, 0);
+            const half2_t s2 = as_half2(sA), b2 = as_half2(bA);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              tot[j][e] = __builtin_fmaf((float)s2[e >> 1], acc[e] - corr[e], __builtin_fmaf((float)b2[e >> 1], xsum[e], tot[j][e]));
+          } else {
+            float4_t accA = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int L = 0; L < 2; ++L)
+#pragma unroll
+              for (int w = 0; w < 4; ++w) {
+                accA = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[L][w], raw_codes(wq[L][w], kMaskLo, kMaskHi, kMagicLo, kMagicHi),
+                                                              accA, 0, 0, 0);
+                accB = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[L + 2][w], raw_codes(wq[L + 2][w], kMaskLo, kMaskHi, kMagicLo, kMagicHi),
+                                                              accB, 0, 0, 0);
+              }
+            float4_t cA, xA, cB, xB;  // group sums of this lane's accumulator rows, halves A and B
+            asm volatile("ds_read_b128 %0, %1 offset:0" : "=v"(cA) : "v"(table_rd));
+            asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(xA) : "v"(table_rd));
+            asm volatile("ds_read_b128 %0, %1 offset:128" : "=v"(cB) : "v"(table_rd));
+            asm volatile("ds_read_b128 %0, %1 offset:144" : "=v"(xB) : "v"(table_rd));
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(cA), "+v"(xA), "+v"(cB), "+v"(xB));
+            const float sa = (float)as_half2(sA)[0], sb = (float)as_half2(sB)[0];
+            const float ba = (float)as_half2(bA)[0], bb = (float)as_half2(bB)[0];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float t = __builtin_fmaf(ba, xA[e], tot[j][e]);
+              t = __builtin_fmaf(bb, xB[e], t);
+              t = __builtin_fmaf(sa, accA[e] - cA[e], t);
+              tot[j][e] = __builtin_fmaf(sb, accB[e] - cB[e], t);
+            }
           }
         }
       }
-      // ---- drop the partial sums into this wave's mailbox once the reducer has emptied it
-      while (lds_load(&ctl->consumed) < q) __builtin_amdgcn_s_sleep(1);
-      if (r < MCAP) {
+      // ---- add up the groups: within the lane (MC 2: rows e and e + 2 are the same batch row),
+      // then over the four slices kc; lanes kc == 0 drop the result into this wave's mailbox once
+      // the reducer has emptied it
+      float out[PR][MC];
 #pragma unroll
-        for (int j = 0; j < kPassRows; ++j)
-          if (j < nj) *reinterpret_cast<float4_t *>(mail + wave * kMailBytes + ((j * 4 + kc) * MCAP + r) * 16) = acc[j];
+      for (int j = 0; j < PR; ++j)
+#pragma unroll
+        for (int m = 0; m < MC; ++m) {
+          float v = MC == 2 ? tot[j][m] + tot[j][m + 2] : tot[j][m];
+          v += lane_read(v, lane ^ 16);
+          v += lane_read(v, lane ^ 32);
+          out[j][m] = v;
+        }
+      while (lds_load(&ctl->consumed) < q) __builtin_amdgcn_s_sleep(1);
+      if (kc == 0) {
+#pragma unroll
+        for (int j = 0; j < PR; ++j)
+          if (j < nj) {
+#pragma unroll
+            for (int m = 0; m < MC; ++m) mail[wave * kMailFloats + (j * MC + m) * 16 + r] = out[j][m];
+          }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the deposit is in LDS before it is counted
       if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -409,9 +576,9 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
 }  // namespace
 
 // (external linkage: the host takes its address for hipFuncSetAttribute)
-template <int MCAP, int NS>
-__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int *status) {
-  gemv_stream_body<MCAP, NS>(reinterpret_cast<const Entry *>(entries), n_entries, status);
+template <int MC, int NS>
+__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int first_entry, int *status) {
+  gemv_stream_body<MC, NS>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status);
 }
 
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
@@ -421,9 +588,9 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   for (int64_t i = 0; i < count && supported; ++i) {
     const gq_gemv_desc &d = host[i];
     if (d.m_rows > max_m) max_m = d.m_rows;
-    supported = d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.m_rows >= 1 && d.m_rows <= 4 &&
-                d.n_out >= 1 && ((uintptr_t)d.x % 16) == 0 && ((uintptr_t)d.packed % 16) == 0 &&
-                ((uintptr_t)d.scale % 16) == 0 && ((uintptr_t)d.bias % 16) == 0;
+    supported = d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.k_in <= (1 << 24) && d.m_rows >= 1 &&
+                d.m_rows <= 4 && d.n_out >= 1 && d.n_out <= (1 << 22) && ((uintptr_t)d.x % 16) == 0 &&
+                ((uintptr_t)d.packed % 16) == 0 && ((uintptr_t)d.scale % 16) == 0 && ((uintptr_t)d.bias % 16) == 0;
   }
   if (!supported || option_gemv_variant() == 3) {
     // any other shape: one launch per entry; stream order provides every dependency
@@ -438,8 +605,9 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
-  static int cu_count[64] = {0};
-  if (dev < 0 || dev >= 64) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
+  constexpr int kMaxDevices = 64;
+  static int cu_count[kMaxDevices] = {0};
+  if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
   if (cu_count[dev] == 0) {
     int n = 0;
     e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
@@ -447,25 +615,27 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     cu_count[dev] = n;
   }
   const int grid = cu_count[dev] < kMaxGroups ? cu_count[dev] : kMaxGroups;  // one workgroup per compute unit, all resident together
-#define GQ_STREAM(MCAP, NS)                                                                                   \
+#define GQ_STREAM(MC, NS)                                                                                     \
   do {                                                                                                        \
     constexpr int lds_bytes =                                                                                 \
-        kWaves * (NS * kItemBytes + MCAP * 1024) + kMaxEntries * 64 + kWaves * kPassRows * 4 * MCAP * 16 + 64;  \
+        kWaves * (NS * kItemBytes + MC * 1024) + kMaxEntries * 64 + kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
+        kWaves * 256;                                                                                         \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
-    auto kern = gemv_stream_kernel<MCAP, NS>;                                                                 \
-    static bool configured = false;                                                                           \
-    if (!configured) {                                                                                        \
+    auto kern = gemv_stream_kernel<MC, NS>;                                                                   \
+    static bool configured[kMaxDevices] = {false};                                                            \
+    if (!configured[dev]) {                                                                                   \
       e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
                               lds_bytes);                                                                     \
       if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
-      configured = true;                                                                                      \
+      configured[dev] = true;                                                                                 \
     }                                                                                                         \
     for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
       const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
-      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status);                     \
+      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, (int)first, status);      \
     }                                                                                                         \
   } while (0)
-  GQ_STREAM(4, 3);
+  if (max_m <= 2) GQ_STREAM(2, 3);
+  else GQ_STREAM(4, 3);
 #undef GQ_STREAM
   return check_launch("gemv_stream_kernel");
 }

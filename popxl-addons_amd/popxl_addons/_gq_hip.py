@@ -104,9 +104,11 @@ def set_option(name, value):
 class GemvSequence:
     """A list of decode GEMVs run by one `gq_gemv_sequence_f16` call (see include/gq_hip.h).
 
-    add(x, packed, scale, bias, y, out_bias=None, wait_previous=False) appends an entry from torch
-    tensors on the GPU (kept alive by this object); run() enqueues the whole list on the current
-    stream.  `status` is a device int32 the kernel sets to 1 if it gave up waiting.
+    add(x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None) appends an
+    entry from torch tensors on the GPU (kept alive by this object) and returns its index; the entry
+    starts after every earlier entry (wait_previous) or after entries 0..wait_for have completed.
+    run() enqueues the whole list on the current stream.  `status` is a device int32 the kernel
+    sets to 1 if it gave up waiting.
     """
 
     def __init__(self, device):
@@ -115,7 +117,7 @@ class GemvSequence:
         self.device = device
         self.dtype = np.dtype(
             [("x", "<u8"), ("packed", "<u8"), ("scale", "<u8"), ("bias", "<u8"), ("out_bias", "<u8"), ("y", "<u8"),
-             ("m_rows", "<i4"), ("n_out", "<i4"), ("k_in", "<i4"), ("group_size", "<i4"), ("wait_previous", "<i4"),
+             ("m_rows", "<i4"), ("n_out", "<i4"), ("k_in", "<i4"), ("group_size", "<i4"), ("wait_entries", "<i4"),
              ("reserved", "<i4")]
         )
         assert self.dtype.itemsize == 72  # sizeof(gq_gemv_desc)
@@ -125,19 +127,24 @@ class GemvSequence:
         self._dev = None
         self.status = None
 
-    def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False):
+    def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None):
         m_rows, k_in = x.shape
         n_out, n_groups, n_ids = packed.shape
         assert y.shape == (m_rows, n_out) and n_groups * n_ids * 4 == k_in
         for t in (x, packed, scale, bias, y):
             assert t.is_cuda and t.is_contiguous()
+        index = len(self.entries)
+        wait_entries = index if wait_previous else (0 if wait_for is None else int(wait_for) + 1)
+        if not 0 <= wait_entries <= index:
+            raise ValueError(f"entry {index} cannot wait for entry {wait_for}")
         self.entries.append(
             (x.data_ptr(), packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
              0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, n_ids * 4,
-             1 if wait_previous else 0, 0)
+             wait_entries, 0)
         )
         self.keep.append((x, packed, scale, bias, y, out_bias))
         self._host = None
+        return index
 
     def _finalise(self):
         import numpy as np

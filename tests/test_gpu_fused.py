@@ -254,3 +254,61 @@ def test_gemv_sequence_fallback_and_graph(hip, device, oracle):
         assert int(seq2.status.item()) == 0
         for o, w_ in zip(outs, want):
             assert torch.equal(o, w_)
+
+
+@pytest.mark.parametrize("m_rows", [1, 3])
+def test_gemv_sequence_wait_for_earlier_entry(hip, device, oracle, m_rows):
+    """Declared dependencies (`wait_entries`): two layers of a parallel decoder block.  q, k, v and
+    up read the layer input; o waits for v only (up keeps streaming meanwhile), down waits for up,
+    and the next layer's projections wait for everything.  Every output equals the single-call
+    GEMV on the same device inputs, bit for bit or within tolerance of the oracle."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    hidden, ffn = 1024, 4096
+    rng = np.random.default_rng(77)
+    seq = GemvSequence(device)
+
+    def weight(n_out, k_in):
+        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        return tuple(to_dev(a, device) for a in group_quantize_compress_numpy(w, 64))
+
+    def out(n):
+        return torch.full((m_rows, n), float("nan"), dtype=torch.float16, device=device)
+
+    x = to_dev(activations(m_rows, hidden, 5), device)
+    plan = []  # (entry index, x tensor, weights, y tensor)
+    last = None
+    for layer in range(2):
+        ys = {name: out(hidden) for name in ("q", "k", "v", "o", "down")}
+        ys["up"] = out(ffn)
+        idx = {}
+        for name in ("q", "k", "v", "up"):
+            w = weight(ffn if name == "up" else hidden, hidden)
+            idx[name] = seq.add(x, *w, ys[name], wait_for=last if name == "q" else None)
+            plan.append((idx[name], x, w, ys[name]))
+        w = weight(hidden, hidden)
+        idx["o"] = seq.add(ys["v"], *w, ys["o"], wait_for=idx["v"])
+        plan.append((idx["o"], ys["v"], w, ys["o"]))
+        w = weight(hidden, ffn)
+        idx["down"] = seq.add(ys["up"], *w, ys["down"], wait_for=idx["up"])
+        plan.append((idx["down"], ys["up"], w, ys["down"]))
+        x, last = ys["down"], idx["down"]  # next layer reads `down`; waiting for it covers o as well
+    with pytest.raises(ValueError):
+        seq.add(x, *weight(hidden, hidden), out(hidden), wait_for=len(seq.entries))  # cannot wait for itself
+
+    for _ in range(3):
+        for _, _, _, y in plan:
+            y.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        for i, x_in, (p, s, b), y in plan:
+            single = torch.empty_like(y)
+            hip.call("gq_gemv_f16", x_in.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0,
+                     single.data_ptr(), y.shape[1], x_in.shape[1], 64, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            yy, ss = y.cpu().numpy(), single.cpu().numpy()
+            assert np.isfinite(yy).all(), i
+            assert normalised_error(yy, ss.astype(np.float32)) <= 2e-3, i  # same inputs, other summation order
+            w_dec = oracle.np_decompress(p.cpu().numpy(), s.cpu().numpy(), b.cpu().numpy())
+            assert normalised_error(yy, oracle.np_linear(x_in.cpu().numpy(), w_dec, None)) <= TOL, i

@@ -55,6 +55,20 @@ def test_abi_version_and_error_text_without_gpu():
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_set_option", b"no_such_option", 1)
     assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED
+    # sequence descriptors are validated on the host copy: an entry cannot wait for itself
+    import numpy as np
+
+    desc = np.zeros(2, dtype=np.dtype([("ptrs", "<u8", 6), ("ints", "<i4", 6)]))
+    assert desc.dtype.itemsize == 72
+    desc["ptrs"] = [[16, 16, 16, 16, 0, 16]] * 2
+    desc["ints"] = [[1, 8, 64, 64, 0, 0], [1, 8, 64, 64, 2, 0]]  # m_rows n_out k_in group_size wait_entries reserved
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE and "wait_entries" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", 0, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
+    _gq_hip.call("gq_gemv_sequence_f16", 0, 0, 0, None, None)  # empty sequence
     # zero-sized problems succeed without touching a device
     _gq_hip.call("gq_decompress_f16", 0, 0, 0, 0, 0, 4, 4, None)
     _gq_hip.call("gq_gemv_f16", 0, 0, 0, 0, 0, 0, 0, 8, 64, 64, None)
