@@ -89,11 +89,13 @@ constexpr int kAuxDeviceCoherent = (1 << 0) | (1 << 4);
 
 // LDS words shared by the waves of a workgroup
 struct Control {
-  unsigned deposited;  // mailbox deposits so far (8 per pass)
-  unsigned consumed;   // passes whose mailboxes the reducer has read
-  unsigned ready;      // entries known to be complete on the whole device
-  unsigned failed;     // the poller gave up
+  unsigned deposited[2];  // mailbox deposits so far, passes of even and of odd number (8 per pass)
+  unsigned consumed;      // passes whose mailboxes the reducer has read
+  unsigned ready;         // entries known to be complete on the whole device
+  unsigned failed;        // the poller gave up
+  unsigned targets[4];    // bit w - 1 set: some entry waits for the first w entries (kMaxEntries bits)
 };
+static_assert(sizeof(Control) <= 64, "control block");
 
 __device__ __forceinline__ unsigned lds_load(const unsigned *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -127,7 +129,8 @@ __device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint3
 // where the target builtins and inline assembly do not exist.)
 //
 // Waves 0..7 compute; they never meet at a workgroup barrier.  After the last chunk of a pass a
-// wave drops its 16 x m partial sums into its mailbox and goes on with the next pass or entry.
+// wave drops its 16 x m partial sums into its mailbox (two sets, used by passes in turn, so a wave
+// may run a pass ahead of the slowest) and goes on with the next pass or entry.
 // Wave 8, the reducer, adds the eight mailboxes in a fixed order, stores y and, for entries that
 // somebody waits for, publishes the workgroup's progress.  Wave 9, the poller, watches the
 // progress words of all workgroups and publishes in LDS how many entries are complete everywhere;
@@ -150,7 +153,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   const int G = gridDim.x, b = blockIdx.x;
   CachedEntry *cache = reinterpret_cast<CachedEntry *>(lds + kWaves * kWaveBytes);
   float *mail = reinterpret_cast<float *>(lds + kWaves * kWaveBytes + kMaxEntries * 64);
-  Control *ctl = reinterpret_cast<Control *>(mail + kWaves * kMailFloats);
+  Control *ctl = reinterpret_cast<Control *>(mail + 2 * kWaves * kMailFloats);  // two sets of mailboxes
   // MC == 4 only: per wave, the group sums of the current x chunk, [half][kc][corr e0..3, xsum e0..3]
   // (registers are short in that variant)
   float *table = reinterpret_cast<float *>(ctl) + 16 + wave * 64;
@@ -173,25 +176,41 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     c.publish = 0;
     cache[i] = c;
   }
-  if (tid == 0) *ctl = Control{0u, 0u, 0u, 0u};
+  if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
   __syncthreads();
   // completion is reported only where an entry waits for it (a report costs the reducer a round
   // trip to memory)
   for (int i = tid; i < n_entries; i += kThreadsAll) {
     const int w = cache[i].wait;
-    if (w > 0) cache[w - 1].publish = 1;
+    if (w > 0) {
+      cache[w - 1].publish = 1;
+      atomicOr(&ctl->targets[(w - 1) >> 5], 1u << ((w - 1) & 31));
+    }
   }
   __syncthreads();
 
   // ============================================================================ poller
   if (wave == kWaves + 1) {
-    int last_waited = 0;  // the largest count anybody waits for
-    for (int d = 1; d < n_entries; ++d) last_waited = max(last_waited, (int)cache[d].wait);
-    // one 16-byte device-coherent load per lane covers 256 workgroups; the minimum over all of them
-    // is the number of entries complete everywhere
+    // the counts somebody waits for, in increasing order: the next one after `ready`
+    const unsigned t0 = (unsigned)uni((int)ctl->targets[0]), t1 = (unsigned)uni((int)ctl->targets[1]);
+    const unsigned t2 = (unsigned)uni((int)ctl->targets[2]), t3 = (unsigned)uni((int)ctl->targets[3]);
+    auto next_target = [&](unsigned ready) -> unsigned {  // smallest waited-for count > ready, 0 if none
+      const unsigned words[4] = {t0, t1, t2, t3};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        unsigned bits = words[w];
+        if (ready >= 32u * (w + 1)) continue;
+        if (ready > 32u * w) bits &= ~0u << (ready - 32u * w);
+        if (bits) return 32u * w + (unsigned)__builtin_ctz(bits) + 1u;
+      }
+      return 0u;
+    };
+    // one 16-byte device-coherent load per lane covers 256 workgroups; a count is complete
+    // everywhere when every workgroup's progress word has reached it
     unsigned ready = 0, spins = 0;
+    unsigned target = next_target(0u);
     const int rounds = (G + 255) >> 8;
-    while (ready < (unsigned)last_waited) {
+    while (target) {
       unsigned lo = 0xffffffffu;
       for (int k = 0; k < rounds; ++k) {
         const int first = (k * 64 + lane) * 4;
@@ -204,10 +223,13 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         for (int i = 0; i < 4; ++i)
           if (first + i < G) lo = min(lo, v[i]);
       }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) lo = min(lo, (unsigned)__shfl_xor((int)lo, off, 64));
-      if (lo > ready) {
-        ready = lo;
+      bool advanced = false;
+      while (target && __builtin_amdgcn_ballot_w64(lo < target) == 0) {  // no lane below the target
+        ready = target;
+        target = next_target(ready);
+        advanced = true;
+      }
+      if (advanced) {
         if (lane == 0) __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         spins = 0;
       } else if (++spins > kSpinLimit) {  // some workgroup is not running: give up, let everybody finish
@@ -230,13 +252,14 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       const half_t *out_bias = cache[d].out_bias;
       for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
         const int nj = min(PR, nrb - pass * PR);
-        while (lds_load(&ctl->deposited) < (q + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
+        while (lds_load(&ctl->deposited[q & 1]) < ((q >> 1) + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
+        const float *box = mail + (q & 1) * kWaves * kMailFloats;
         // one sum per (row block j, batch row m, output n): consecutive lanes, consecutive n
         for (int t = lane; t < nj * MC * 16; t += 64) {
           const int n16 = t & 15, m = (t >> 4) % MC, j = t / (16 * MC);
           float sum = 0.f;
 #pragma unroll
-          for (int w = 0; w < kWaves; ++w) sum += mail[w * kMailFloats + t];
+          for (int w = 0; w < kWaves; ++w) sum += box[w * kMailFloats + t];
           const int n = (b + (pass * PR + j) * G) * 16 + n16;
           if (m < m_rows && n < n_out) {
             if (out_bias) sum += (float)out_bias[n];
@@ -557,17 +580,17 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           v += lane_read(v, lane ^ 32);
           out[j][m] = v;
         }
-      while (lds_load(&ctl->consumed) < q) __builtin_amdgcn_s_sleep(1);
+      while (lds_load(&ctl->consumed) + 1 < q) __builtin_amdgcn_s_sleep(1);  // the box of pass q - 2 is free
       if (kc == 0) {
 #pragma unroll
         for (int j = 0; j < PR; ++j)
           if (j < nj) {
 #pragma unroll
-            for (int m = 0; m < MC; ++m) mail[wave * kMailFloats + (j * MC + m) * 16 + r] = out[j][m];
+            for (int m = 0; m < MC; ++m) mail[((q & 1) * kWaves + wave) * kMailFloats + (j * MC + m) * 16 + r] = out[j][m];
           }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the deposit is in LDS before it is counted
-      if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited[q & 1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
   wait_vm<0>();
@@ -618,7 +641,7 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
 #define GQ_STREAM(MC, NS)                                                                                     \
   do {                                                                                                        \
     constexpr int lds_bytes =                                                                                 \
-        kWaves * (NS * kItemBytes + MC * 1024) + kMaxEntries * 64 + kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
+        kWaves * (NS * kItemBytes + MC * 1024) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
         kWaves * 256;                                                                                         \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
     auto kern = gemv_stream_kernel<MC, NS>;                                                                   \
