@@ -39,6 +39,7 @@ constexpr int kItemOps = 6;             // direct-to-LDS loads per item: 4 packe
 // for them); the variant for 4 batch rows has fewer registers to spare
 constexpr int pass_rows(int mc) { return mc == 2 ? 4 : 2; }
 constexpr unsigned kSpinLimit = 1u << 18;
+constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, batch row)
 
 // Progress of the running sequence on this device.  Every workgroup publishes the number of
 // entries it has completed in its own word (plain device-scope stores: 256 read-modify-writes of
@@ -145,7 +146,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   static_assert(MC == 2 || MC == 4, "batch capacity");
   constexpr int PR = pass_rows(MC);
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  constexpr int kWaveBytes = NS * kItemBytes + MC * 1024;
+  constexpr int kWaveBytes = NS * kItemBytes + kStageBytes;
   constexpr int kMailFloats = PR * MC * 16;  // per wave: [row block][m][n]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
@@ -396,6 +397,8 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   }
   const half_t *x_loaded = nullptr;  // the operands in registers belong to (x_loaded, chunk x_chunk)
   int x_chunk = -1, x_k = 0, x_m = 0;
+  const half_t *st_x = nullptr;  // the stage holds this wave's chunk of EVERY phase of (st_x, st_k, st_m)
+  int st_k = 0, st_m = 0;
   unsigned known_ready = 0;  // entries this wave has seen complete on the whole device
 
   for (int d = 0; d < n_entries; ++d) {
@@ -407,6 +410,25 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       // every workgroup has finished the first `need` entries (published by the poller)
       while ((known_ready = lds_load(&ctl->ready)) < need && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
       x_loaded = nullptr;
+      st_x = nullptr;
+    }
+    // an entry with several phases whose x chunks all fit the stage fetches them in one go: one
+    // drain of the ring per entry instead of one per phase
+    const bool fits_all = phases > 1 && phases * m_rows * 1024 <= kStageBytes;
+    bool staged = fits_all && st_x == x && st_k == k_in && st_m == m_rows;
+    if (fits_all && !staged && nrb > 0) {
+      for (int phase = 0; phase < phases; ++phase) {
+        const int chunk = phase * kWaves + wave;
+        if (chunk * 512 >= k_in) continue;
+        for (int m = 0; m < m_rows; ++m)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
+                                           xstage + (phase * m_rows + m) * 1024, 16, 0, kAuxDeviceCoherent);
+      }
+      wait_vm<0>();
+      st_x = x;
+      st_k = k_in;
+      st_m = m_rows;
+      staged = true;
     }
     for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
       const int nj = min(PR, nrb - pass * PR);
@@ -418,11 +440,16 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         if (chunk * 512 >= k_in) continue;
         // ---- A operands and group sums of this chunk (kept when the previous entry used the same x)
         const bool reload_x = !(x_loaded == x && x_chunk == chunk && x_k == k_in && x_m == m_rows);
+        const bool drained = reload_x && !staged;
         if (reload_x) {
-          for (int m = 0; m < m_rows; ++m)
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
-                                             xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
-          wait_vm<0>();  // x is the youngest load: everything in flight lands with it
+          if (!staged) {
+            for (int m = 0; m < m_rows; ++m)
+              __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
+                                               xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
+            wait_vm<0>();  // x is the youngest load: everything in flight lands with it
+            st_x = nullptr;
+          }
+          const uint32_t xs_rd = x_rd + (staged ? phase * m_rows * 1024 : 0);
           const bool active = a_match && a_m < m_rows;
           constexpr int HALVES = MC == 2 ? 1 : 2;
           float part_sum[HALVES], part_corr[HALVES];
@@ -435,7 +462,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             for (int j = 0; j < 4; ++j)
               asm volatile("ds_read_b128 %0, %1 offset:%2"
                            : "=v"(xq[j])
-                           : "v"(x_rd + a_m * 1024 + (4 * load + kc) * 64), "n"(j * 16));
+                           : "v"(xs_rd + a_m * 1024 + (4 * load + kc) * 64), "n"(j * 16));
             asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xq[0]), "+v"(xq[1]), "+v"(xq[2]), "+v"(xq[3]));
             float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -492,7 +519,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         for (int j = 0; j < PR; ++j) {
           if (j >= nj) break;
           // ---- this item's loads are older than those of the n_ahead - 1 items issued after it
-          if (!reload_x || j > 0) {
+          if (!drained || j > 0) {
             if (n_ahead >= 4) wait_vm<3 * kItemOps>();
             else if (n_ahead == 3) wait_vm<2 * kItemOps>();
             else if (n_ahead == 2) wait_vm<kItemOps>();
@@ -641,7 +668,7 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
 #define GQ_STREAM(MC, NS)                                                                                     \
   do {                                                                                                        \
     constexpr int lds_bytes =                                                                                 \
-        kWaves * (NS * kItemBytes + MC * 1024) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
+        kWaves * (NS * kItemBytes + kStageBytes) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
         kWaves * 256;                                                                                         \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
     auto kern = gemv_stream_kernel<MC, NS>;                                                                   \
