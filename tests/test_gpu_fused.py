@@ -312,3 +312,40 @@ def test_gemv_sequence_wait_for_earlier_entry(hip, device, oracle, m_rows):
             assert normalised_error(yy, ss.astype(np.float32)) <= 2e-3, i  # same inputs, other summation order
             w_dec = oracle.np_decompress(p.cpu().numpy(), s.cpu().numpy(), b.cpu().numpy())
             assert normalised_error(yy, oracle.np_linear(x_in.cpu().numpy(), w_dec, None)) <= TOL, i
+
+
+def test_gemv_sequence_longer_than_one_launch(hip, device, oracle):
+    """More entries than one launch of the persistent kernel holds (128): the sequence continues
+    in a second launch, and dependencies that reach back across the boundary hold."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    rng = np.random.default_rng(21)
+    seq = GemvSequence(device)
+    n_entries, width = 140, 512
+    x0 = activations(2, width, 9)
+    weights, outs = [], []
+    x_in = to_dev(x0, device)
+    for i in range(n_entries):
+        w = rng.normal(0, 1.0 / np.sqrt(width), (width, width)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        y = torch.full((2, width), float("nan"), dtype=torch.float16, device=device)
+        # every third entry starts a new chain from x0; the others read their predecessor
+        chained = i % 3 != 0
+        seq.add(x_in if chained else to_dev(x0, device), to_dev(packed, device), to_dev(scale, device),
+                to_dev(bias, device), y, wait_for=i - 1 if chained else None)
+        weights.append((packed, scale, bias, chained))
+        outs.append(y)
+        x_in = y
+    for _ in range(2):
+        for y in outs:
+            y.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        prev = None
+        for i, ((packed, scale, bias, chained), y) in enumerate(zip(weights, outs)):
+            yy = y.cpu().numpy()
+            assert np.isfinite(yy).all(), i
+            x_host = prev if chained else x0
+            assert normalised_error(yy, oracle.np_linear(x_host, oracle.np_decompress(packed, scale, bias), None)) <= TOL, i
+            prev = yy
