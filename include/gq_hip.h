@@ -43,6 +43,12 @@ extern "C" {
 #define GQ_ERR_UNSUPPORTED (-4)  /* well-formed, but outside what the kernels cover */
 #define GQ_ERR_NO_DEVICE (-5)    /* no usable gfx950 device / code object */
 
+/* Epilogues of the fused matmul entry points: applied to sum + out_bias in binary32 before the
+ * result is rounded to binary16. */
+#define GQ_ACT_NONE 0
+#define GQ_ACT_RELU 1
+#define GQ_ACT_GELU_TANH 2 /* 0.5 v (1 + tanh(sqrt(2/pi) (v + 0.044715 v^3))) */
+
 /* ABI version of the loaded library (GQ_ABI_VERSION it was built with). */
 int gq_abi_version(void);
 
@@ -114,6 +120,16 @@ int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, con
                   int64_t k_in, int64_t group_size, void *stream);
 
 /*
+ * gq_linear_f16 with an activation fused into the epilogue: y = act(x w^T + out_bias), the step
+ * that follows the up-projection of a decoder's feed-forward block.  No counterpart in the
+ * reference (LinearGQ.build ends at the bias add, popxl_addons/layers/linear_gq.py:102-109, and
+ * the activation is a separate op of the model); `activation` is one of GQ_ACT_*.
+ */
+int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                      const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                      int64_t k_in, int64_t group_size, int32_t activation, void *stream);
+
+/*
  * A sequence of decode GEMVs (a layer stack) as one call.  No counterpart in the reference, where
  * a model is a chain of LinearGQ.build calls (popxl_addons/layers/linear_gq.py:99-109) compiled
  * into one static device program; this entry point is the analogue for a chain of gq_gemv_f16
@@ -144,7 +160,7 @@ typedef struct gq_gemv_desc {
   uint16_t *y;              /* [m_rows, n_out] binary16 */
   int32_t m_rows, n_out, k_in, group_size;
   int32_t wait_entries;     /* entries [0, wait_entries) complete before this one starts */
-  int32_t reserved;         /* 0 */
+  int32_t activation;       /* GQ_ACT_*: epilogue of this entry */
 } gq_gemv_desc;
 
 int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,

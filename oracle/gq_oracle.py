@@ -167,9 +167,25 @@ def np_compress(t, group_size, dim=-1):
     return packed, scale, lo
 
 
-def np_linear(x, w_dec, out_bias=None):
-    """fp32 matmul over the decompressed weight (tests/integration/layers/test_linear_gq.py:18-30,52)."""
+def np_linear(x, w_dec, out_bias=None, activation=None):
+    """fp32 matmul over the decompressed weight (tests/integration/layers/test_linear_gq.py:18-30,52),
+    optionally followed by np_activation."""
     y = x.astype(np.float32) @ w_dec.astype(np.float32).T
     if out_bias is not None:
         y = y + out_bias.astype(np.float32)
-    return y
+    return np_activation(y, activation)
+
+
+def np_activation(v, activation):
+    """The epilogues of the fused entry points, in binary64.  No counterpart in the reference's
+    path (its layer ends at the bias add, popxl_addons/layers/linear_gq.py:102-109): "relu" is
+    max(v, 0); "gelu_tanh" is the tanh form of GELU, 0.5 v (1 + tanh(sqrt(2/pi) (v + 0.044715 v^3))).
+    Pinned in tests/test_oracle_pinned.py by scalar evaluation with math.tanh and by identities."""
+    if activation in (None, "none"):
+        return v
+    v64 = np.asarray(v, dtype=np.float64)
+    if activation == "relu":
+        return np.maximum(v64, 0.0)
+    if activation == "gelu_tanh":
+        return 0.5 * v64 * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (v64 + 0.044715 * v64**3)))
+    raise ValueError(f"unknown activation {activation!r}")

@@ -116,7 +116,7 @@ int gq_gemv_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   if (m_rows > 16)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_f16: m_rows=%lld exceeds 16; use gq_gemm_f16",
                     (long long)m_rows);
-  return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+  return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, GQ_ACT_NONE,
                          (hipStream_t)stream);
 }
 
@@ -126,7 +126,7 @@ int gq_gemm_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   const int rc = gq::check_linear_args("gq_gemm_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
                                        k_in, group_size);
   if (rc <= 0) return rc;
-  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, GQ_ACT_NONE,
                          (hipStream_t)stream);
 }
 
@@ -136,10 +136,21 @@ int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, con
   const int rc = gq::check_linear_args("gq_linear_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
                                        k_in, group_size);
   if (rc <= 0) return rc;
+  return gq_linear_act_f16(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, GQ_ACT_NONE, stream);
+}
+
+int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                      const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                      int64_t group_size, int32_t activation, void *stream) {
+  const int rc = gq::check_linear_args("gq_linear_act_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
+                                       k_in, group_size);
+  if (rc <= 0) return rc;
+  if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_act_f16: unknown activation %d", (int)activation);
   if (m_rows <= 16)
-    return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+    return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
                            (hipStream_t)stream);
-  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
                          (hipStream_t)stream);
 }
 
@@ -160,6 +171,9 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
     if (d.m_rows > 16)
       return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld has m_rows=%d > 16", (long long)i,
                       d.m_rows);
+    if (d.activation < GQ_ACT_NONE || d.activation > GQ_ACT_GELU_TANH)
+      return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld has unknown activation %d", (long long)i,
+                      d.activation);
     if (d.wait_entries < 0 || d.wait_entries > i)
       return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: entry %lld has wait_entries=%d outside [0, %lld]",
                       (long long)i, d.wait_entries, (long long)i);

@@ -25,15 +25,28 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
+// Epilogue applied to sum + out_bias before the result is rounded to binary16 (GQ_ACT_* of the C ABI).
+__device__ __forceinline__ float apply_activation(float v, int act) {
+  if (act == GQ_ACT_RELU) return fmaxf(v, 0.f);
+  if (act == GQ_ACT_GELU_TANH) {
+    const float u = 0.7978845608028654f * (v + 0.044715f * (v * v * v));
+    return 0.5f * v * (1.f + tanhf(u));
+  }
+  return v;
+}
+
 // Launchers implemented next to their kernels.
 int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
                       int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed, hipStream_t stream);
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, hipStream_t stream);
+                int64_t group_size, int act, hipStream_t stream);
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, hipStream_t stream);
+                int64_t group_size, int act, hipStream_t stream);
+int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                             const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                             int64_t k_in, int64_t group_size, int act, hipStream_t stream);
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
                          hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,

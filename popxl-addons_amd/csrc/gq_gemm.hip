@@ -7,10 +7,6 @@
 
 namespace gq {
 
-int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
-                             const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
-                             int64_t k_in, int64_t group_size, hipStream_t stream);
-
 namespace {
 
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -52,7 +48,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const half_t *__restrict
                                                         const half_t *__restrict__ scale,
                                                         const half_t *__restrict__ bias,
                                                         const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                        int n_out, int k_in, int gs_shift) {
+                                                        int n_out, int k_in, int gs_shift, int act) {
   __shared__ __attribute__((aligned(16))) half_t As[BM][LDK];
   __shared__ __attribute__((aligned(16))) half_t Bs[BN][LDK];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -133,7 +129,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const half_t *__restrict
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)(acc[i][j][e] + ob);
+        if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)apply_activation(acc[i][j][e] + ob, act);
       }
     }
 }
@@ -265,7 +261,7 @@ template <int WM, int WN, int FM, int FN, int XS>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
-    int gs_shift) {
+    int gs_shift, int act) {
   using S = Pipe2Shape<WM, WN, FM, FN, XS>;
   constexpr int NW = S::NW, TM = S::TM, TN = S::TN, TILE_M = S::TILE_M, TILE_N = S::TILE_N;
   constexpr int A_OPS = S::A_OPS, OPS = S::OPS;
@@ -471,12 +467,13 @@ __device__ __forceinline__ void gemm_pipe2_body(
       half_t *dst = y + (int64_t)(m0 + wm * TM + i * 32 + 4 * h) * n_out + n;
       if (interior) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) dst[(int64_t)(8 * (e >> 2) + (e & 3)) * n_out] = (half_t)(acc[i][f][e] + ob);
+        for (int e = 0; e < 16; ++e)
+          dst[(int64_t)(8 * (e >> 2) + (e & 3)) * n_out] = (half_t)apply_activation(acc[i][f][e] + ob, act);
       } else if (n < n_out) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int m = m0 + wm * TM + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-          if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)(acc[i][f][e] + ob);
+          if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)apply_activation(acc[i][f][e] + ob, act);
         }
       }
     }
@@ -493,8 +490,8 @@ template <int WM, int WN, int FM, int FN, int XS, int OCC>
 __global__ __launch_bounds__(WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
                                                                   const half_t *scale, const half_t *bias,
                                                                   const half_t *out_bias, half_t *y, int n_out,
-                                                                  int k_in, int gs_shift) {
-  gemm_pipe2_body<WM, WN, FM, FN, XS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift);
+                                                                  int k_in, int gs_shift, int act) {
+  gemm_pipe2_body<WM, WN, FM, FN, XS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act);
 }
 
 namespace {
@@ -502,7 +499,7 @@ namespace {
 template <int WM, int WN, int FM, int FN, int XS, int OCC>
 int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int gs_shift,
-                 hipStream_t stream) {
+                 int act, hipStream_t stream) {
   using S = Pipe2Shape<WM, WN, FM, FN, XS>;
   constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
   static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
@@ -519,7 +516,7 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
   kern<<<grid, dim3(WM * WN * 64), lds_bytes, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
-      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift);
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act);
   return check_launch("gemm_pipe2_kernel");
 }
 
@@ -527,16 +524,16 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
 
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, hipStream_t stream) {
+                int64_t group_size, int act, hipStream_t stream) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % BK == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
   if (!fast_ok || option_gemm_variant() == 1)
-    return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, stream);
+    return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
   const int variant = option_gemm_variant();
 #define GQ_PIPE2(WM, WN, FM, FN, XS, OCC) \
-  launch_pipe2<WM, WN, FM, FN, XS, OCC>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, stream)
+  launch_pipe2<WM, WN, FM, FN, XS, OCC>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
   if (variant != 2 && (k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
     int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 2);
@@ -555,7 +552,7 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   gemm_tile_kernel<<<grid, dim3(256), 0, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
-      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift);
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act);
   return check_launch("gemm_tile_kernel");
 }
 

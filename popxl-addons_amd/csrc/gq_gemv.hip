@@ -34,7 +34,7 @@ template <int NWAVES, int R, int GS, bool FULL>
 __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
-    int gs_shift) {
+    int gs_shift, int act) {
   __shared__ float4_t partial[NWAVES][R][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kc = lane >> 4;
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
         if (n < n_out) {
           float v = sum[e];
           if (out_bias) v += (float)out_bias[n];
-          y[(int64_t)m * n_out + n] = (half_t)v;
+          y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
         }
       }
     }
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
                                                            const half_t *__restrict__ scale,
                                                            const half_t *__restrict__ bias,
                                                            const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                           int n_out, int k_in, int group_size) {
+                                                           int n_out, int k_in, int group_size, int act) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= n_out) return;
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
       for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
       if (lane == 0) {
         if (out_bias) v += (float)out_bias[row];
-        y[(int64_t)m * n_out + row] = (half_t)v;
+        y[(int64_t)m * n_out + row] = (half_t)apply_activation(v, act);
       }
     }
   }
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, hipStream_t stream) {
+                int64_t group_size, int act, hipStream_t stream) {
   const int variant = option_gemv_variant();
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
@@ -224,7 +224,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 #define GQ_GEMV_ARGS                                                                                      \
   reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),                    \
-      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act
 #define GQ_GEMV_LAUNCH(NW, R, GS, FULL) \
   gemv_mfma_kernel<NW, R, GS, FULL><<<dim3(blocks), dim3(NW * 64), 0, stream>>>(GQ_GEMV_ARGS)
 #define GQ_GEMV_BY_R(NW, GS, FULL)                      \
@@ -252,21 +252,21 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   gemv_generic_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, packed, reinterpret_cast<const half_t *>(scale),
       reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias),
-      reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, (int)group_size);
+      reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, (int)group_size, act);
   return check_launch("gemv_generic_kernel");
 }
 
 // Any m_rows through the generic kernel, 16 batch rows per launch (fallback of the GEMM entry).
 int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                              const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
-                             int64_t k_in, int64_t group_size, hipStream_t stream) {
+                             int64_t k_in, int64_t group_size, int act, hipStream_t stream) {
   const unsigned blocks = (unsigned)((n_out + 3) / 4);
   for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
     const int m = (int)(m_rows - m0 < 16 ? m_rows - m0 : 16);
     gemv_generic_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(
         reinterpret_cast<const half_t *>(x) + m0 * k_in, m, packed, reinterpret_cast<const half_t *>(scale),
         reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias),
-        reinterpret_cast<half_t *>(y) + m0 * n_out, (int)n_out, (int)k_in, (int)group_size);
+        reinterpret_cast<half_t *>(y) + m0 * n_out, (int)n_out, (int)k_in, (int)group_size, act);
   }
   return check_launch("gemv_generic_kernel");
 }

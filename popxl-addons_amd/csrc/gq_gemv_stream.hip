@@ -56,7 +56,7 @@ struct Entry {  // = gq_gemv_desc
   const half_t *bias;
   const half_t *out_bias;
   half_t *y;
-  int32_t m_rows, n_out, k_in, group_size, wait_entries, reserved;
+  int32_t m_rows, n_out, k_in, group_size, wait_entries, activation;
 };
 static_assert(sizeof(Entry) == sizeof(gq_gemv_desc), "descriptor layout");
 
@@ -79,7 +79,8 @@ struct CachedEntry {
   int n_out, k_in;
   short m_rows, wait;  // wait: entries of this launch that must be complete before this one starts
   short nrb;           // row blocks owned by this workgroup
-  short publish;       // somebody waits for exactly this entry and its predecessors: report its completion
+  char publish;        // somebody waits for exactly this entry and its predecessors: report its completion
+  char act;            // GQ_ACT_* epilogue
 };
 static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
 constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
@@ -175,6 +176,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     const int rb = (e.n_out + 15) >> 4;
     c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
     c.publish = 0;
+    c.act = (char)e.activation;
     cache[i] = c;
   }
   if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
@@ -251,6 +253,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), n_out = uni(cache[d].n_out);
       half_t *y = cache[d].y;
       const half_t *out_bias = cache[d].out_bias;
+      const int act = uni(cache[d].act);
       for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
         const int nj = min(PR, nrb - pass * PR);
         while (lds_load(&ctl->deposited[q & 1]) < ((q >> 1) + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
@@ -264,7 +267,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           const int n = (b + (pass * PR + j) * G) * 16 + n16;
           if (m < m_rows && n < n_out) {
             if (out_bias) sum += (float)out_bias[n];
-            const half_t hv = (half_t)sum;
+            const half_t hv = (half_t)apply_activation(sum, act);
             // device-scope store: written through to where every compute unit reads it
             __hip_atomic_store(reinterpret_cast<unsigned short *>(y) + (int64_t)m * n_out + n,
                                __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -647,7 +650,7 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     for (int64_t i = 0; i < count; ++i) {
       const gq_gemv_desc &d = host[i];
       const int rc = launch_gemv(d.x, d.m_rows, d.packed, d.scale, d.bias, d.out_bias, d.y, d.n_out, d.k_in,
-                                 d.group_size, stream);
+                                 d.group_size, d.activation, stream);
       if (rc != GQ_OK) return rc;
     }
     return GQ_OK;

@@ -16,6 +16,18 @@ GQ_ERR_BAD_SHAPE = -2
 GQ_ERR_MISALIGNED = -3
 GQ_ERR_UNSUPPORTED = -4
 GQ_ERR_NO_DEVICE = -5
+GQ_ACT_NONE, GQ_ACT_RELU, GQ_ACT_GELU_TANH = 0, 1, 2
+ACTIVATIONS = {None: GQ_ACT_NONE, "none": GQ_ACT_NONE, "relu": GQ_ACT_RELU, "gelu_tanh": GQ_ACT_GELU_TANH}
+
+
+def activation_code(activation):
+    """GQ_ACT_* of an activation given by name (None, "relu", "gelu_tanh") or by code."""
+    if isinstance(activation, int) and activation in ACTIVATIONS.values():
+        return activation
+    try:
+        return ACTIVATIONS[activation]
+    except (KeyError, TypeError):
+        raise ValueError(f"unknown activation {activation!r}; expected one of {sorted(k for k in ACTIVATIONS if k)}") from None
 
 # every symbol declared in include/gq_hip.h
 EXPORTS = (
@@ -27,6 +39,7 @@ EXPORTS = (
     "gq_gemv_f16",
     "gq_gemm_f16",
     "gq_linear_f16",
+    "gq_linear_act_f16",
     "gq_gemv_sequence_f16",
     "gq_compress_f16",
 )
@@ -75,6 +88,8 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, p]
         fn.restype = ctypes.c_int
+    lib.gq_linear_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p]
+    lib.gq_linear_act_f16.restype = ctypes.c_int
     lib.gq_gemv_sequence_f16.argtypes = [p, p, i64, p, p]
     lib.gq_gemv_sequence_f16.restype = ctypes.c_int
     lib.gq_compress_f16.argtypes = [p, p, p, p, p, i64, i64, i64, p]
@@ -104,7 +119,7 @@ def set_option(name, value):
 class GemvSequence:
     """A list of decode GEMVs run by one `gq_gemv_sequence_f16` call (see include/gq_hip.h).
 
-    add(x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None) appends an
+    add(x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None, activation=None) appends an
     entry from torch tensors on the GPU (kept alive by this object) and returns its index; the entry
     starts after every earlier entry (wait_previous) or after entries 0..wait_for have completed.
     run() enqueues the whole list on the current stream.  `status` is a device int32 the kernel
@@ -118,7 +133,7 @@ class GemvSequence:
         self.dtype = np.dtype(
             [("x", "<u8"), ("packed", "<u8"), ("scale", "<u8"), ("bias", "<u8"), ("out_bias", "<u8"), ("y", "<u8"),
              ("m_rows", "<i4"), ("n_out", "<i4"), ("k_in", "<i4"), ("group_size", "<i4"), ("wait_entries", "<i4"),
-             ("reserved", "<i4")]
+             ("activation", "<i4")]
         )
         assert self.dtype.itemsize == 72  # sizeof(gq_gemv_desc)
         self.entries = []
@@ -127,7 +142,7 @@ class GemvSequence:
         self._dev = None
         self.status = None
 
-    def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None):
+    def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None, activation=None):
         m_rows, k_in = x.shape
         n_out, n_groups, n_ids = packed.shape
         assert y.shape == (m_rows, n_out) and n_groups * n_ids * 4 == k_in
@@ -140,7 +155,7 @@ class GemvSequence:
         self.entries.append(
             (x.data_ptr(), packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
              0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, n_ids * 4,
-             wait_entries, 0)
+             wait_entries, activation_code(activation))
         )
         self.keep.append((x, packed, scale, bias, y, out_bias))
         self._host = None

@@ -99,9 +99,14 @@ class LinearGQ:
 
     # --------------------------------------------------------------------------------- build
 
-    def build(self, x):
-        """y = x @ decompress(weight) (+ bias), linear_gq.py:99-109.  x: float16 [..., in] on the GPU."""
+    def build(self, x, activation=None):
+        """y = x @ decompress(weight) (+ bias), linear_gq.py:99-109.  x: float16 [..., in] on the GPU.
+
+        activation (None, "relu", "gelu_tanh") is an addition to the reference's signature: the
+        epilogue is fused into the kernel for dim=0 and applied by torch otherwise."""
         import torch
+
+        act = _gq_hip.activation_code(activation)
 
         if not x.is_cuda:
             raise RuntimeError("LinearGQ runs on the GPU only: move x to a HIP device")
@@ -121,7 +126,7 @@ class LinearGQ:
             with torch.cuda.device(x.device):
                 y = torch.empty((x2.shape[0], self.out_features), dtype=torch.float16, device=x.device)
                 _gq_hip.call(
-                    "gq_linear_f16",
+                    "gq_linear_act_f16",
                     x2.data_ptr(),
                     x2.shape[0],
                     v.weight_compressed.data.data_ptr(),
@@ -132,6 +137,7 @@ class LinearGQ:
                     self.out_features,
                     in_features,
                     self.group_size,
+                    act,
                     torch.cuda.current_stream(x.device).cuda_stream,
                 )
             return y.reshape(*x.shape[:-1], self.out_features)
@@ -144,6 +150,10 @@ class LinearGQ:
         y = x @ w
         if b is not None:
             y = y + b
+        if act == _gq_hip.GQ_ACT_RELU:
+            y = torch.relu(y)
+        elif act == _gq_hip.GQ_ACT_GELU_TANH:
+            y = torch.nn.functional.gelu(y.float(), approximate="tanh").to(y.dtype)
         return y
 
     __call__ = build

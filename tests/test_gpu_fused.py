@@ -349,3 +349,53 @@ def test_gemv_sequence_longer_than_one_launch(hip, device, oracle):
             x_host = prev if chained else x0
             assert normalised_error(yy, oracle.np_linear(x_host, oracle.np_decompress(packed, scale, bias), None)) <= TOL, i
             prev = yy
+
+
+@pytest.mark.parametrize("activation,code", [("relu", 1), ("gelu_tanh", 2)])
+@pytest.mark.parametrize("m_rows", [1, 8, 40, 300])
+def test_fused_activation_epilogue(hip, device, oracle, activation, code, m_rows):
+    """gq_linear_act_f16: the activation is applied to sum + out_bias in every kernel the dispatch
+    reaches (MFMA GEMV, generic GEMV, pipelined GEMM, tile GEMM)."""
+    for n_out, k_in, gs in ((520, 1024, 64), (96, 192, 64), (24, 40, 20)):
+        x, packed, scale, bias, ob, _ = _case(oracle, n_out, k_in, gs, m_rows, 71, True)
+        y_ref = oracle.np_linear(x, oracle.np_decompress(packed, scale, bias), ob, activation)
+        xd, pd, sd, bd, od = (to_dev(a, device) for a in (x, packed, scale, bias, ob))
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        hip.call("gq_linear_act_f16", xd.data_ptr(), m_rows, pd.data_ptr(), sd.data_ptr(), bd.data_ptr(), od.data_ptr(),
+                 y.data_ptr(), n_out, k_in, gs, code, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        yy = y.cpu().numpy()
+        assert np.isfinite(yy).all()
+        assert normalised_error(yy, y_ref) <= TOL, (n_out, k_in, gs)
+        if activation == "relu":
+            assert (yy >= 0).all()
+
+
+@pytest.mark.parametrize("m_rows", [1, 4, 8])
+def test_gemv_sequence_activation(hip, device, oracle, m_rows):
+    """Per-entry activation in a sequence: up-projection with GELU feeding the down-projection
+    (persistent kernel for m_rows <= 4, one launch per entry above)."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    hidden, ffn = 512, 2048
+    rng = np.random.default_rng(91)
+    x = activations(m_rows, hidden, 3)
+    w_up = rng.normal(0, 1.0 / np.sqrt(hidden), (ffn, hidden)).astype(np.float16)
+    w_down = rng.normal(0, 1.0 / np.sqrt(ffn), (hidden, ffn)).astype(np.float16)
+    b_up = rng.normal(0, 0.5, (ffn,)).astype(np.float16)
+    up = group_quantize_compress_numpy(w_up, 64)
+    down = group_quantize_compress_numpy(w_down, 64)
+    seq = GemvSequence(device)
+    y_up = torch.full((m_rows, ffn), float("nan"), dtype=torch.float16, device=device)
+    y_down = torch.full((m_rows, hidden), float("nan"), dtype=torch.float16, device=device)
+    first = seq.add(to_dev(x, device), *(to_dev(a, device) for a in up), y_up, to_dev(b_up, device), activation="gelu_tanh")
+    seq.add(y_up, *(to_dev(a, device) for a in down), y_down, wait_for=first, activation="relu")
+    for _ in range(2):
+        y_up.fill_(float("nan"))
+        y_down.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        got_up, got_down = y_up.cpu().numpy(), y_down.cpu().numpy()
+        assert normalised_error(got_up, oracle.np_linear(x, oracle.np_decompress(*up), b_up, "gelu_tanh")) <= TOL
+        assert normalised_error(got_down, oracle.np_linear(got_up, oracle.np_decompress(*down), None, "relu")) <= TOL

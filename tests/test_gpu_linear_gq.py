@@ -155,3 +155,24 @@ def test_fuse_rejects_mismatched_layers(hip, device):
         LinearGQ.fuse([a, c])
     with pytest.raises(ValueError):
         LinearGQ.fuse([])
+
+
+@pytest.mark.parametrize("dim", [0, -1])
+@pytest.mark.parametrize("activation", ["relu", "gelu_tanh"])
+def test_linear_gq_activation(hip, device, oracle, dim, activation):
+    """LinearGQ.build(x, activation=...): fused epilogue for dim=0, torch epilogue otherwise."""
+    in_features, out_features, group_size = 256, 384, 64
+    torch.manual_seed(4)
+    nn_layer = torch.nn.Linear(in_features, out_features)
+    layer = LinearGQ(out_features, bias=True, group_size=group_size, dim=dim)
+    variables = layer.init_variables(in_features, torch.float16, device)
+    mapping = LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=dim)
+    layer.load_weights(mapping)
+    x = torch.randn((5, in_features), device=device, dtype=torch.float16)
+    plain = layer(x).float().cpu().numpy()
+    got = layer.build(x, activation=activation).float().cpu().numpy()
+    want = oracle.np_activation(plain, activation)
+    # the fused path activates the unrounded sum, the reference point here the fp16-rounded one
+    assert normalised_error(got, want) <= 2e-3
+    with pytest.raises(ValueError):
+        layer.build(x, activation="swish")

@@ -69,6 +69,17 @@ def test_abi_version_and_error_text_without_gpu():
         _gq_hip.call("gq_gemv_sequence_f16", 0, 16, 2, None, None)
     assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
     _gq_hip.call("gq_gemv_sequence_f16", 0, 0, 0, None, None)  # empty sequence
+    # an unknown activation is rejected before anything is launched
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_act_f16", 16, 1, 16, 16, 16, 0, 16, 8, 64, 64, 7, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "activation" in str(e.value)
+    desc["ints"] = [[1, 8, 64, 64, 0, 0], [1, 8, 64, 64, 1, 9]]
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "activation" in str(e.value)
+    assert _gq_hip.activation_code("gelu_tanh") == _gq_hip.GQ_ACT_GELU_TANH and _gq_hip.activation_code(None) == 0
+    with pytest.raises(ValueError):
+        _gq_hip.activation_code("swish")
     # zero-sized problems succeed without touching a device
     _gq_hip.call("gq_decompress_f16", 0, 0, 0, 0, 0, 4, 4, None)
     _gq_hip.call("gq_gemv_f16", 0, 0, 0, 0, 0, 0, 0, 8, 64, 64, None)

@@ -190,3 +190,24 @@ def test_linear_oracle_is_a_matmul(oracle):
     np.testing.assert_allclose(oracle.c_linear(x, w, ob), ref, rtol=1e-6, atol=1e-7)
     np.testing.assert_allclose(oracle.np_linear(x, w, ob), ref, rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(oracle.c_linear(x, w), x.astype(np.float64) @ w.astype(np.float64).T, rtol=1e-6, atol=1e-7)
+
+
+def test_activation_oracle(oracle):
+    """The epilogue restatement against scalar evaluation and against what the functions must
+    satisfy: gelu(v) - gelu(-v) = v, gelu(0) = 0, gelu -> identity / 0 far from the origin, and the
+    known value of the tanh form at 1 (0.841192 to six places; the erf form gives 0.841345)."""
+    import math
+
+    grid = np.linspace(-8, 8, 1601)
+    g = oracle.np_activation(grid, "gelu_tanh")
+    want = [0.5 * v * (1.0 + math.tanh(math.sqrt(2.0 / math.pi) * (v + 0.044715 * v * v * v))) for v in grid]
+    np.testing.assert_allclose(g, want, rtol=0, atol=1e-15)
+    np.testing.assert_allclose(g - g[::-1], grid, atol=1e-12)
+    assert oracle.np_activation(np.array([0.0]), "gelu_tanh")[0] == 0.0
+    assert abs(oracle.np_activation(np.array([1.0]), "gelu_tanh")[0] - 0.841192) < 5e-7
+    assert abs(g[-1] - 8.0) < 1e-9 and abs(g[0]) < 1e-9
+    r = oracle.np_activation(grid, "relu")
+    assert np.array_equal(r, np.where(grid > 0, grid, 0.0))
+    assert oracle.np_activation(grid, None) is grid
+    with pytest.raises(ValueError):
+        oracle.np_activation(grid, "swish")
