@@ -439,12 +439,16 @@ __device__ __forceinline__ void gemm_pipe2_body(
       }
       if (i >= 2) {
 #pragma unroll
-        for (int f = 0; f < FN; ++f) dequant_piece<FM - 2>(i - 2, wq_next[f][0], s2n[f], z2n[f], st[f]);
+        for (int f = 0; f < FN; ++f) dequant_piece<(FM > 2 ? FM - 2 : 1)>(i - 2, wq_next[f][0], s2n[f], z2n[f], st[f]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int i = 0; i < FM; ++i) asm volatile("" : : "v"(a[1][i]));
+    if (FM == 2) {  // no MFMA group left to hide the expansion behind
+#pragma unroll
+      for (int f = 0; f < FN; ++f) dequant_piece<1>(0, wq_next[f][0], s2n[f], z2n[f], st[f]);
+    }
 #pragma unroll
     for (int f = 0; f < FN; ++f) {
       b_cur[f] = dequant_result(st[f]);
@@ -536,14 +540,15 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   launch_pipe2<WM, WN, FM, FN, XS, OCC>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
   if (variant != 2 && (k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 2);
-    if (variant >= 30 && variant <= 34) shape = variant - 30;
+    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 5);
+    if (variant >= 30 && variant <= 35) shape = variant - 30;
     switch (shape) {
       case 0: return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
       case 1: return GQ_PIPE2(1, 4, 8, 1, 3, 1);  // 256 x 128, 4 waves of 256 x 32
       case 2: return GQ_PIPE2(1, 4, 4, 1, 3, 2);  // 128 x 128, 4 waves of 128 x 32, two workgroups per CU
       case 3: return GQ_PIPE2(1, 4, 4, 2, 3, 2);  // 128 x 256, 4 waves of 128 x 64, two workgroups per CU
-      default: return GQ_PIPE2(2, 2, 4, 2, 3, 1);  // 256 x 128, 4 waves of 128 x 64
+      case 4: return GQ_PIPE2(2, 2, 4, 2, 3, 1);  // 256 x 128, 4 waves of 128 x 64
+      default: return GQ_PIPE2(2, 2, 2, 1, 3, 2);  // 128 x 64, 4 waves of 64 x 32: a workgroup on every compute unit at n_out = 16384
     }
   }
 #undef GQ_PIPE2

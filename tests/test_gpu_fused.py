@@ -110,9 +110,9 @@ def test_gemm_edge_shapes(hip, device, oracle, n_out, k_in, gs, m_rows):
             assert normalised_error(y, y_ref) <= TOL, (entry, with_bias)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 30, 31, 32, 33, 34])
+@pytest.mark.parametrize("variant", [1, 2, 30, 31, 32, 33, 34, 35])
 def test_gemm_every_kernel_shape(hip, device, oracle, variant):
-    """Each tile shape of the pipelined kernel (30..34), the LDS-staged tile kernel (2) and the
+    """Each tile shape of the pipelined kernel (30..35), the LDS-staged tile kernel (2) and the
     generic kernel (1) on ragged problems, including a weight with an odd number of groups per row
     (which the pipelined kernel hands to the tile kernel)."""
     try:
