@@ -283,6 +283,9 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           __hip_atomic_store(&g_progress[b], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+    // a sequence without dependencies has not touched the progress words
+    const unsigned any_target = ctl->targets[0] | ctl->targets[1] | ctl->targets[2] | ctl->targets[3];
+    if (uni((int)any_target) == 0) return;
     // the last workgroup out clears the progress words: by then every poller has seen all it needs
     wait_vm<0>();  // this workgroup's last progress word is in memory before it counts itself out
     unsigned last = 0;
