@@ -85,9 +85,10 @@ struct CachedEntry {
 static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
 constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
 
-// cache policy of a direct-to-LDS load: sc0 | sc1 = coherent at device scope (bypasses the L1 of
-// the compute unit and the non-coherent part of the L2 of its XCD)
-constexpr int kAuxDeviceCoherent = (1 << 0) | (1 << 4);
+// cache policy of a direct-to-LDS load: sc1 = device (agent) scope, the policy the compiler gives an
+// agent-scope atomic load; it pairs with the agent-scope stores of y and of the progress words
+// (sc0 | sc1, system scope, costs another 2 % of a pass)
+constexpr int kAuxDeviceCoherent = 1 << 4;
 
 // LDS words shared by the waves of a workgroup
 struct Control {
@@ -218,7 +219,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       for (int k = 0; k < rounds; ++k) {
         const int first = (k * 64 + lane) * 4;
         uint4_t v;
-        asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)"
+        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
                      : "=v"(v)
                      : "v"(g_progress + first)
                      : "memory");
