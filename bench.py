@@ -199,6 +199,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     #   parallel block     attention and feed-forward read the same layer input (the 6B model of
     #                      these shapes is built that way): order q k v up o down; q waits for the
     #                      previous layer, o for v (up streams meanwhile), down for up
+    #   ... fused qkv       the parallel block with q, k, v as one 12288 x 4096 entry: 112 entries per pass
     #   no waits           no dependencies: the streaming rate of the kernel alone, not a decoder
     def sequential(seq):
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
@@ -214,12 +215,25 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                 idx[role] = seq.add(xs[k_in], p, s, b, ys[role], None, wait_for=wait_for)
             last = idx[5]
 
+    def parallel_fused_qkv(seq):
+        # the same, with q, k and v stacked into one [3 * hidden x hidden] entry (LinearGQ.fuse): 112 entries
+        last = None
+        for layer in range(n_layers):
+            q, k, v, o, up, down = (mats[layer * 6 + role] for role in range(6))
+            a = seq.add(xs[hidden], *fused_qkv[layer], y_qkv, None, wait_for=last)
+            b_ = seq.add(xs[hidden], *up[2:], ys[4], None)
+            seq.add(xs[hidden], *o[2:], ys[3], None, wait_for=a)
+            last = seq.add(xs[ffn], *down[2:], ys[5], None, wait_for=b_)
+
     def free(seq):
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
             seq.add(xs[k_in], p, s, b, ys[i % 6], None)
 
+    fused_qkv = [tuple(torch.cat([mats[layer * 6 + role][2 + part] for role in range(3)], dim=0).contiguous()
+                       for part in range(3)) for layer in range(n_layers)]
+    y_qkv = torch.empty((m_rows, 3 * hidden), dtype=torch.float16, device=device)
     for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
-                       ("sequence_no_waits", free)):
+                       ("sequence_parallel_block_fused_qkv", parallel_fused_qkv), ("sequence_no_waits", free)):
         seq = hip.GemvSequence(device)
         fill(seq)
         ms = time_launches(lambda _: seq.run(), passes, warmup)
@@ -311,7 +325,8 @@ def main():
         for m in (1, 4):
             r = bench_stack(hip, device, m, passes=20, warmup=3)
             extra["stack"].append(r)
-            for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block", "sequence_no_waits"):
+            for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block",
+                         "sequence_parallel_block_fused_qkv", "sequence_no_waits"):
                 log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
                     f"({r[mode]['hbm_frac']:.1%})")
             torch.cuda.empty_cache()
