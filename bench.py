@@ -101,6 +101,31 @@ def bench_decompress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384
     return {"ms": ms, "bytes": bytes_per_launch, "gbs": bytes_per_launch / ms / 1e6, "sets": sets}
 
 
+def bench_compress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384):
+    """Device-side packer on the configuration-2 weight: reads 2 B, writes 0.5 + 4/gs B per element."""
+    import torch
+
+    sets = []
+    for s in range(n_sets):
+        w = make_weight(rows, cols, 100 + s, True, device)
+        n_groups = cols // GROUP
+        sets.append((w, torch.empty((rows, n_groups, GROUP // 4), dtype=torch.uint16, device=device),
+                     torch.empty((rows, n_groups, 1), dtype=torch.float16, device=device),
+                     torch.empty((rows, n_groups, 1), dtype=torch.float16, device=device)))
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    stream = stream_handle()
+
+    def step(i):
+        w, p, s, b = sets[i % n_sets]
+        hip.call("gq_compress_f16", w.data_ptr(), p.data_ptr(), s.data_ptr(), b.data_ptr(), flag.data_ptr(), rows,
+                 cols // GROUP, GROUP, stream)
+
+    ms = time_launches(step, steps, warmup)
+    nbytes = rows * cols * (2.0 + 0.5 + 4.0 / GROUP)
+    return {"rows": rows, "cols": cols, "us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / ms / 1e6,
+            "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+
+
 def cpu_baseline_decompress(sets, rows_sample=4096):
     """The numpy restatement of the reference's decompress (oracle/), timed on the host cores on one
     full 4096 x 16384 weight, best of 3.  numpy's elementwise passes run on one thread."""
@@ -305,6 +330,11 @@ def main():
     del dec["sets"]
     torch.cuda.empty_cache()
 
+    if args.only == "all":
+        r = bench_compress(hip, device, 100, 10)
+        extra["compress"] = r
+        log(f"  compress 4096x16384: {r['us']:.1f} us, {r['gbs']:.0f} GB/s algorithmic ({r['hbm_frac']:.1%} of HBM peak)")
+        torch.cuda.empty_cache()
     if args.only in ("gemv", "all"):
         extra["gemv"] = []
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):

@@ -508,12 +508,16 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
   constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
   static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
   auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC>;
-  static bool configured = false;  // same value every time: a benign race
-  if (!configured) {
+  // the attribute belongs to the (function, device) pair; same value every time: a benign race
+  constexpr int kMaxDevices = 64;
+  static bool configured[kMaxDevices] = {false};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_NO_DEVICE, "no current device");
+  if (!configured[dev]) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute(lds=%d): %s", lds_bytes, hipGetErrorString(e));
-    configured = true;
+    configured[dev] = true;
   }
   const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M));
   if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_gemm_f16: m_rows=%lld too large", (long long)m_rows);
