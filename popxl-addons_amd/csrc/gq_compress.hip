@@ -19,10 +19,22 @@ constexpr int kThreads = 256;
 
 __device__ __forceinline__ bool nonfinite_bits(uint32_t h) { return (h & 0x7c00u) == 0x7c00u; }
 
-__device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, half_t scale) {
-  if ((float)scale == 0.f) return 0u;  // constant group: undefined in the reference, code 0 here
+// f16(diff / scale), correctly rounded, from a reciprocal shared by the group: one Newton step on
+// the fp32 product.  Why that is enough: the residual e = diff - scale * t is exact (an fma of
+// 11-bit by 24-bit operands whose result cancels down to a few bits), so t2 = t + e * r lies
+// within one fp32 ulp of the true quotient, while a quotient of two 11-bit significands is at
+// least 2^-22 (relative, in [1, 2)) away from every fp16 rounding boundary -- four fp32 ulps.  No
+// boundary can lie between t2 and the quotient, so rounding t2 rounds the quotient.
+__device__ __forceinline__ half_t divide(half_t diff, float scale_f32, float recip) {
+  const float d = (float)diff;
+  const float t = d * recip;
+  const float e = __builtin_fmaf(-scale_f32, t, d);
+  return (half_t)__builtin_fmaf(e, recip, t);
+}
+
+__device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float scale_f32, float recip) {
   const half_t diff = v - lo;
-  const half_t quot = (half_t)((float)diff / (float)scale);
+  const half_t quot = divide(diff, scale_f32, recip);
   int c = (int)__builtin_rintf((float)quot);
   c = c < 0 ? 0 : (c > 15 ? 15 : c);  // no effect wherever the reference is well defined
   return (uint32_t)c;
@@ -63,9 +75,13 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
   }
   const half_t range = hi - lo;
   const half_t sc = (half_t)((float)range / 15.0f);
+  // scale 0 (a constant group, or a range too small for fp16): every code is 0; dividing by 1 gives
+  // that without a branch, because every difference is then below 2^-20
+  const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
+  const float recip = __builtin_amdgcn_rcpf(sc32);
   uint32_t c[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) c[e] = quantize(v[e], lo, sc);
+  for (int e = 0; e < 8; ++e) c[e] = quantize(v[e], lo, sc32, recip);
   const uint32_t w0 = (c[0] << 12) | (c[1] << 8) | (c[2] << 4) | c[3];
   const uint32_t w1 = (c[4] << 12) | (c[5] << 8) | (c[6] << 4) | c[7];
   if (live) {
@@ -99,9 +115,11 @@ __global__ __launch_bounds__(kThreads) void compress_generic_kernel(const half_t
   const half_t sc = (half_t)((float)range / 15.0f);
   scale[g] = sc;
   bias[g] = lo;
+  const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
+  const float recip = __builtin_amdgcn_rcpf(sc32);
   for (int i = 0; i < group_size / 4; ++i) {
     uint32_t w = 0;
-    for (int j = 0; j < 4; ++j) w = (w << 4) | quantize(src[4 * i + j], lo, sc);
+    for (int j = 0; j < 4; ++j) w = (w << 4) | quantize(src[4 * i + j], lo, sc32, recip);
     packed[g * (group_size / 4) + i] = (uint16_t)w;
   }
   if (bad && flag) *flag = 1;
