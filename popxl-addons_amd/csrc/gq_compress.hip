@@ -27,7 +27,7 @@ __device__ __forceinline__ bool nonfinite_bits(uint32_t h) { return (h & 0x7c00u
 // boundary can lie between t2 and the quotient, so rounding t2 rounds the quotient.
 __device__ __forceinline__ half_t divide(half_t diff, float scale_f32, float recip) {
   const float d = (float)diff;
-  const float t = d * recip;
+  const float t = __builtin_fmaf(d, recip, 0.f);  // the product, as a mixed-precision fma that reads diff as fp16
   const float e = __builtin_fmaf(-scale_f32, t, d);
   return (half_t)__builtin_fmaf(e, recip, t);
 }
@@ -42,6 +42,23 @@ __device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float scale_f3
 
 // LANES lanes share one group; each lane holds 8 consecutive elements (one 16-byte load) and
 // writes the two uint16 words made from them as one 32-bit store.  group_size = 8 * LANES.
+// The kernel is bound by instruction issue, not by HBM, so the work is done two elements per
+// instruction wherever a packed fp16 form exists (the roundings are those of the scalar forms).
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+
+// packed minimum / maximum as single instructions (the generic builtins first quieten their
+// operands with two more)
+__device__ __forceinline__ half2_t pk_min(half2_t a, half2_t b) {
+  half2_t r;
+  asm("v_pk_min_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ half2_t pk_max(half2_t a, half2_t b) {
+  half2_t r;
+  asm("v_pk_max_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
 template <int LANES>
 __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__restrict__ t, uint32_t *__restrict__ packed,
                                                             half_t *__restrict__ scale, half_t *__restrict__ bias,
@@ -50,47 +67,55 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
   const bool live = item < n_items;
   uint4_t q = {0u, 0u, 0u, 0u};
   if (live) q = __builtin_nontemporal_load(t + item);
-  half_t v[8];
-  bool bad = false;
+  half2_t h[4];
+  ushort2_t exponents = {0, 0};  // maximum of the exponent fields: 0x7c00 = Inf or NaN seen
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
-    const uint32_t w = q[d];
-    bad |= nonfinite_bits(w) | nonfinite_bits(w >> 16);
-    const half2_t h = __builtin_bit_cast(half2_t, w);
-    v[2 * d] = h[0];
-    v[2 * d + 1] = h[1];
+    const uint32_t w = q[d];  // (a bit cast straight from a vector element reads element 0)
+    h[d] = __builtin_bit_cast(half2_t, w);
+    const uint32_t e = w & 0x7c007c00u;
+    exponents = __builtin_elementwise_max(exponents, __builtin_bit_cast(ushort2_t, e));
   }
-  half_t hi = v[0], lo = v[0];
-#pragma unroll
-  for (int e = 1; e < 8; ++e) {
-    hi = v[e] > hi ? v[e] : hi;
-    lo = v[e] < lo ? v[e] : lo;
-  }
-  // the whole wave executes the shuffles; items of one group are LANES consecutive lanes
+  const half2_t mx = pk_max(pk_max(h[0], h[1]), pk_max(h[2], h[3]));
+  const half2_t mn = pk_min(pk_min(h[0], h[1]), pk_min(h[2], h[3]));
+  // (min, max) of the group travel through the shuffles as one register; the whole wave executes
+  // them, items of one group are LANES consecutive lanes
+  half2_t p = {mn[0] < mn[1] ? mn[0] : mn[1], mx[0] > mx[1] ? mx[0] : mx[1]};
 #pragma unroll
   for (int off = LANES / 2; off > 0; off >>= 1) {
-    const half_t ohi = (half_t)__shfl_xor((float)hi, off, 64), olo = (half_t)__shfl_xor((float)lo, off, 64);
-    hi = ohi > hi ? ohi : hi;
-    lo = olo < lo ? olo : lo;
+    const half2_t o = __builtin_bit_cast(half2_t, __shfl_xor(__builtin_bit_cast(int, p), off, 64));
+    const half2_t lo2 = pk_min(p, o), hi2 = pk_max(p, o);
+    p = half2_t{lo2[0], hi2[1]};
   }
+  const half_t lo = p[0], hi = p[1];
   const half_t range = hi - lo;
   const half_t sc = (half_t)((float)range / 15.0f);
   // scale 0 (a constant group, or a range too small for fp16): every code is 0; dividing by 1 gives
   // that without a branch, because every difference is then below 2^-20
   const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
   const float recip = __builtin_amdgcn_rcpf(sc32);
-  uint32_t c[8];
+  const half2_t lo_pair = {lo, lo}, fifteen = {(half_t)15.0f, (half_t)15.0f}, magic = {(half_t)1024.0f, (half_t)1024.0f};
+  uint32_t m[4];  // codes of elements (2d, 2d + 1) at bits 3:0 and 19:16
 #pragma unroll
-  for (int e = 0; e < 8; ++e) c[e] = quantize(v[e], lo, sc32, recip);
-  const uint32_t w0 = (c[0] << 12) | (c[1] << 8) | (c[2] << 4) | c[3];
-  const uint32_t w1 = (c[4] << 12) | (c[5] << 8) | (c[6] << 4) | c[7];
+  for (int d = 0; d < 4; ++d) {
+    const half2_t diff = h[d] - lo_pair;
+    half2_t code;
+    code[0] = __builtin_rintf16(divide(diff[0], sc32, recip));
+    code[1] = __builtin_rintf16(divide(diff[1], sc32, recip));
+    code = pk_min(code, fifteen);  // no effect wherever the reference is well defined
+    // 1024 + c has the code in its low mantissa bits
+    const half2_t biased = code + magic;
+    m[d] = __builtin_bit_cast(uint32_t, biased) & 0x000F000Fu;
+  }
+  const uint32_t w0 = ((m[0] << 12) | (m[0] >> 8) | (m[1] << 4) | (m[1] >> 16)) & 0xFFFFu;
+  const uint32_t w1 = ((m[2] << 12) | (m[2] >> 8) | (m[3] << 4) | (m[3] >> 16)) & 0xFFFFu;
   if (live) {
     packed[item] = w0 | (w1 << 16);
     if ((item & (LANES - 1)) == 0) {
       scale[item / LANES] = sc;
       bias[item / LANES] = lo;
     }
-    if (bad && flag) *flag = 1;
+    if (flag && (exponents[0] == 0x7c00 || exponents[1] == 0x7c00)) *flag = 1;
   }
 }
 
