@@ -94,17 +94,16 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
   // that without a branch, because every difference is then below 2^-20
   const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
   const float recip = __builtin_amdgcn_rcpf(sc32);
-  const half2_t lo_pair = {lo, lo}, fifteen = {(half_t)15.0f, (half_t)15.0f}, magic = {(half_t)1024.0f, (half_t)1024.0f};
+  const half2_t lo_pair = {lo, lo}, ceiling = {(half_t)1039.0f, (half_t)1039.0f}, magic = {(half_t)1024.0f, (half_t)1024.0f};
   uint32_t m[4];  // codes of elements (2d, 2d + 1) at bits 3:0 and 19:16
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
     const half2_t diff = h[d] - lo_pair;
-    half2_t code;
-    code[0] = __builtin_rintf16(divide(diff[0], sc32, recip));
-    code[1] = __builtin_rintf16(divide(diff[1], sc32, recip));
-    code = pk_min(code, fifteen);  // no effect wherever the reference is well defined
-    // 1024 + c has the code in its low mantissa bits
-    const half2_t biased = code + magic;
+    const half2_t quot = {divide(diff[0], sc32, recip), divide(diff[1], sc32, recip)};
+    // quot + 1024 rounds to an integer, ties to even (the ulp of fp16 at 1024 is 1): that is
+    // 1024 + rint(quot), with the code in the low mantissa bits.  Codes above 15 are clipped (no
+    // effect wherever the reference is well defined).
+    const half2_t biased = pk_min(quot + magic, ceiling);
     m[d] = __builtin_bit_cast(uint32_t, biased) & 0x000F000Fu;
   }
   const uint32_t w0 = ((m[0] << 12) | (m[0] >> 8) | (m[1] << 4) | (m[1] >> 16)) & 0xFFFFu;
