@@ -250,6 +250,18 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             seq.add(xs[hidden], *o[2:], ys[3], None, wait_for=a)
             last = seq.add(xs[ffn], *down[2:], ys[5], None, wait_for=b_)
 
+    def parallel_fused_qkv_ffn_first(seq):
+        # the same dependencies, entries ordered up, qkv, down, o: each wait names an entry that is
+        # two entries back, so another matrix streams while its result settles; only the step to
+        # the next layer (which needs o and down, both at the end) is exposed
+        last = None
+        for layer in range(n_layers):
+            q, k, v, o, up, down = (mats[layer * 6 + role] for role in range(6))
+            b_ = seq.add(xs[hidden], *up[2:], ys[4], None, wait_for=last)
+            a = seq.add(xs[hidden], *fused_qkv[layer], y_qkv, None)
+            seq.add(xs[ffn], *down[2:], ys[5], None, wait_for=b_)
+            last = seq.add(xs[hidden], *o[2:], ys[3], None, wait_for=a)
+
     def free(seq):
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
             seq.add(xs[k_in], p, s, b, ys[i % 6], None)
@@ -258,7 +270,9 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                        for part in range(3)) for layer in range(n_layers)]
     y_qkv = torch.empty((m_rows, 3 * hidden), dtype=torch.float16, device=device)
     for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
-                       ("sequence_parallel_block_fused_qkv", parallel_fused_qkv), ("sequence_no_waits", free)):
+                       ("sequence_parallel_block_fused_qkv", parallel_fused_qkv),
+                       ("sequence_parallel_block_fused_qkv_ffn_first", parallel_fused_qkv_ffn_first),
+                       ("sequence_no_waits", free)):
         seq = hip.GemvSequence(device)
         fill(seq)
         ms = time_launches(lambda _: seq.run(), passes, warmup)

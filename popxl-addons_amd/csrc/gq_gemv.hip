@@ -208,6 +208,16 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream) {
   const int variant = option_gemv_variant();
+  // Large weights at small batches go through the persistent kernel as a sequence of one: its
+  // pipelined rings beat the one-shot kernel below once the weight is tens of megabytes (measured:
+  // 16384x4096 at one row 14.5 -> 11.7 us). With 3 or 4 rows that holds only for the wide outputs
+  // (4096x16384: 17.2 us one-shot, 18.0 us streamed). Variant 4 forces the route, 2 forbids it.
+  const bool large = n_out * k_in >= ((int64_t)24 << 20) && (m_rows <= 2 || n_out >= 8192);
+  if ((variant == 4 || (variant == 0 && large)) && m_rows <= 4) {
+    const int rc =
+        launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
+    if (rc != GQ_ERR_UNSUPPORTED) return rc;
+  }
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;

@@ -142,9 +142,10 @@ __device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint3
 // Visibility of results between compute units needs no cache flush: y is written with device-scope
 // stores (sc1, write-through to the coherent level), the reducer waits for its stores before it
 // publishes, and x is read with device-coherent loads.
-template <int MC, int NS>
+// SINGLE: the sequence is the one entry `single`, passed by value (no descriptor in memory).
+template <int MC, int NS, bool SINGLE>
 __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries, int first_entry,
-                                                 int *__restrict__ status) {
+                                                 int *__restrict__ status, const Entry single) {
   static_assert(MC == 2 || MC == 4, "batch capacity");
   constexpr int PR = pass_rows(MC);
   extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -162,7 +163,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   float *table = reinterpret_cast<float *>(ctl) + 16 + wave * 64;
 
   for (int i = tid; i < n_entries; i += kThreadsAll) {
-    const Entry e = entries[i];
+    const Entry e = SINGLE ? single : entries[i];
     CachedEntry c;
     c.packed = reinterpret_cast<const char *>(e.packed);
     c.scale = reinterpret_cast<const char *>(e.scale);
@@ -635,7 +636,104 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
 // (external linkage: the host takes its address for hipFuncSetAttribute)
 template <int MC, int NS>
 __global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int first_entry, int *status) {
-  gemv_stream_body<MC, NS>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status);
+  gemv_stream_body<MC, NS, false>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status, Entry{});
+}
+
+// one GEMV through the same body: what gq_gemv_f16 launches for large weights
+template <int MC, int NS>
+__global__ __launch_bounds__(kThreadsAll) void gemv_stream_single_kernel(const gq_gemv_desc desc) {
+  Entry e;
+  e.x = reinterpret_cast<const half_t *>(desc.x);
+  e.packed = reinterpret_cast<const uint4_t *>(desc.packed);
+  e.scale = reinterpret_cast<const half_t *>(desc.scale);
+  e.bias = reinterpret_cast<const half_t *>(desc.bias);
+  e.out_bias = reinterpret_cast<const half_t *>(desc.out_bias);
+  e.y = reinterpret_cast<half_t *>(desc.y);
+  e.m_rows = desc.m_rows;
+  e.n_out = desc.n_out;
+  e.k_in = desc.k_in;
+  e.group_size = desc.group_size;
+  e.wait_entries = 0;
+  e.activation = desc.activation;
+  gemv_stream_body<MC, NS, true>(nullptr, 1, 0, nullptr, e);
+}
+
+namespace {
+
+bool stream_shape_ok(const gq_gemv_desc &d) {
+  return d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.k_in <= (1 << 24) && d.m_rows >= 1 &&
+         d.m_rows <= 4 && d.n_out >= 1 && d.n_out <= (1 << 22) && ((uintptr_t)d.x % 16) == 0 &&
+         ((uintptr_t)d.packed % 16) == 0 && ((uintptr_t)d.scale % 16) == 0 && ((uintptr_t)d.bias % 16) == 0;
+}
+
+constexpr int kMaxDevices = 64;
+
+// one workgroup per compute unit, all resident together; 0 with the error recorded
+int stream_grid(int *dev_out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e)), 0;
+  static int cu_count[kMaxDevices] = {0};
+  if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev), 0;
+  if (cu_count[dev] == 0) {
+    int n = 0;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || n <= 0) return fail((int)e, "cannot query the compute unit count"), 0;
+    cu_count[dev] = n;
+  }
+  *dev_out = dev;
+  return cu_count[dev] < kMaxGroups ? cu_count[dev] : kMaxGroups;
+}
+
+template <int MC, int NS>
+constexpr int stream_lds_bytes() {
+  return kWaves * (NS * kItemBytes + kStageBytes) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +
+         kWaves * 256;
+}
+
+}  // namespace
+
+// One GEMV as a single-entry run of the persistent kernel; GQ_ERR_UNSUPPORTED (without an error
+// text) if the shape is outside it.
+int launch_gemv_streamed(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                         int64_t group_size, int act, hipStream_t stream) {
+  if (m_rows > 4 || n_out > (1 << 22) || k_in > (1 << 24) || group_size != 64) return GQ_ERR_UNSUPPORTED;
+  gq_gemv_desc d;
+  d.x = x;
+  d.packed = packed;
+  d.scale = scale;
+  d.bias = bias;
+  d.out_bias = out_bias;
+  d.y = y;
+  d.m_rows = (int)m_rows;
+  d.n_out = (int)n_out;
+  d.k_in = (int)k_in;
+  d.group_size = (int)group_size;
+  d.wait_entries = 0;
+  d.activation = act;
+  if (!stream_shape_ok(d)) return GQ_ERR_UNSUPPORTED;
+  int dev = 0;
+  const int grid = stream_grid(&dev);
+  if (grid == 0) return GQ_ERR_NO_DEVICE;
+#define GQ_SINGLE(MC, NS)                                                                                     \
+  do {                                                                                                        \
+    constexpr int lds_bytes = stream_lds_bytes<MC, NS>();                                                     \
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
+    auto kern = gemv_stream_single_kernel<MC, NS>;                                                            \
+    static bool configured[kMaxDevices] = {false};                                                            \
+    if (!configured[dev]) {                                                                                   \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                          \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);        \
+      if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
+      configured[dev] = true;                                                                                 \
+    }                                                                                                         \
+    kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(d);                                            \
+  } while (0)
+  if (m_rows <= 2) GQ_SINGLE(2, 3);
+  else GQ_SINGLE(4, 3);
+#undef GQ_SINGLE
+  return check_launch("gemv_stream_single_kernel");
 }
 
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
@@ -643,11 +741,8 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   int max_m = 1;
   bool supported = count <= (1 << 20);
   for (int64_t i = 0; i < count && supported; ++i) {
-    const gq_gemv_desc &d = host[i];
-    if (d.m_rows > max_m) max_m = d.m_rows;
-    supported = d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.k_in <= (1 << 24) && d.m_rows >= 1 &&
-                d.m_rows <= 4 && d.n_out >= 1 && d.n_out <= (1 << 22) && ((uintptr_t)d.x % 16) == 0 &&
-                ((uintptr_t)d.packed % 16) == 0 && ((uintptr_t)d.scale % 16) == 0 && ((uintptr_t)d.bias % 16) == 0;
+    if (host[i].m_rows > max_m) max_m = host[i].m_rows;
+    supported = stream_shape_ok(host[i]);
   }
   if (!supported || option_gemv_variant() == 3) {
     // any other shape: one launch per entry; stream order provides every dependency
@@ -660,29 +755,17 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     return GQ_OK;
   }
   int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
-  constexpr int kMaxDevices = 64;
-  static int cu_count[kMaxDevices] = {0};
-  if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
-  if (cu_count[dev] == 0) {
-    int n = 0;
-    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess || n <= 0) return fail((int)e, "cannot query the compute unit count");
-    cu_count[dev] = n;
-  }
-  const int grid = cu_count[dev] < kMaxGroups ? cu_count[dev] : kMaxGroups;  // one workgroup per compute unit, all resident together
+  const int grid = stream_grid(&dev);
+  if (grid == 0) return GQ_ERR_NO_DEVICE;
 #define GQ_STREAM(MC, NS)                                                                                     \
   do {                                                                                                        \
-    constexpr int lds_bytes =                                                                                 \
-        kWaves * (NS * kItemBytes + kStageBytes) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +   \
-        kWaves * 256;                                                                                         \
+    constexpr int lds_bytes = stream_lds_bytes<MC, NS>();                                                     \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
     auto kern = gemv_stream_kernel<MC, NS>;                                                                   \
     static bool configured[kMaxDevices] = {false};                                                            \
     if (!configured[dev]) {                                                                                   \
-      e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                              lds_bytes);                                                                     \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                          \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);        \
       if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
       configured[dev] = true;                                                                                 \
     }                                                                                                         \

@@ -35,7 +35,7 @@ def _case(oracle, n_out, k_in, gs, m_rows, seed, with_bias):
 
 
 @pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (16384, 4096), (4096, 16384)])
-@pytest.mark.parametrize("m_rows", [1, 4, 8, 16])
+@pytest.mark.parametrize("m_rows", [1, 2, 3, 4, 8, 16])
 def test_gemv_benchmark_shapes(hip, device, oracle, n_out, k_in, m_rows):
     """Benchmark configurations 3 and 5: decode batches on the layer shapes of the 6B stack."""
     for with_bias in (False, True):
@@ -355,8 +355,10 @@ def test_gemv_sequence_longer_than_one_launch(hip, device, oracle):
 @pytest.mark.parametrize("m_rows", [1, 8, 40, 300])
 def test_fused_activation_epilogue(hip, device, oracle, activation, code, m_rows):
     """gq_linear_act_f16: the activation is applied to sum + out_bias in every kernel the dispatch
-    reaches (MFMA GEMV, generic GEMV, pipelined GEMM, tile GEMM)."""
-    for n_out, k_in, gs in ((520, 1024, 64), (96, 192, 64), (24, 40, 20)):
+    reaches (MFMA GEMV, generic GEMV, single GEMV through the persistent kernel, pipelined GEMM,
+    tile GEMM)."""
+    shapes = ((520, 1024, 64), (96, 192, 64), (24, 40, 20)) + (((8192, 4096, 64),) if m_rows == 1 else ())
+    for n_out, k_in, gs in shapes:
         x, packed, scale, bias, ob, _ = _case(oracle, n_out, k_in, gs, m_rows, 71, True)
         y_ref = oracle.np_linear(x, oracle.np_decompress(packed, scale, bias), ob, activation)
         xd, pd, sd, bd, od = (to_dev(a, device) for a in (x, packed, scale, bias, ob))
