@@ -44,9 +44,19 @@ constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, 
 // Progress of the running sequence on this device.  Every workgroup publishes the number of
 // entries it has completed in its own word (plain device-scope stores: 256 read-modify-writes of
 // one counter per entry would serialise at the memory side); the last workgroup to leave the
-// kernel clears the words.
+// kernel clears the words.  Each word has a 128-byte line to itself: with 32 words to a line every
+// store hit a line that all 256 pollers were reading, and the stream of weights lost 4 - 5 us per
+// published entry (measured: polling lines that nobody writes, or writing lines that nobody
+// polls, costs nothing).
+// For the same reason only the pollers of the first kMasters workgroups read those words; each
+// announces the count that is complete everywhere in a word of its own, which the pollers of the
+// workgroups b with b % kMasters equal to its index watch (one more hop for a wait that is
+// exposed, 1/32 of the loads that collide with the stores).
 constexpr int kMaxGroups = 1024;
-__device__ __attribute__((aligned(16))) unsigned int g_progress[kMaxGroups];
+constexpr int kProgressStride = 32;  // words
+constexpr int kMasters = 1;
+__device__ __attribute__((aligned(128))) unsigned int g_progress[kMaxGroups * kProgressStride];
+__device__ __attribute__((aligned(128))) unsigned int g_announced[kMasters * kProgressStride];
 __device__ unsigned int g_exited;  // workgroups that left the kernel
 
 struct Entry {  // = gq_gemv_desc
@@ -96,6 +106,7 @@ struct Control {
   unsigned consumed;      // passes whose mailboxes the reducer has read
   unsigned ready;         // entries known to be complete on the whole device
   unsigned failed;        // the poller gave up
+  unsigned published;     // entries this workgroup has reported complete (progress word written)
   unsigned targets[4];    // bit w - 1 set: some entry waits for the first w entries (kMaxEntries bits)
 };
 static_assert(sizeof(Control) <= 64, "control block");
@@ -181,7 +192,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     c.act = (char)e.activation;
     cache[i] = c;
   }
-  if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
+  if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
   __syncthreads();
   // completion is reported only where an entry waits for it (a report costs the reducer a round
   // trip to memory)
@@ -210,23 +221,40 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       }
       return 0u;
     };
-    // one 16-byte device-coherent load per lane covers 256 workgroups; a count is complete
-    // everywhere when every workgroup's progress word has reached it
+    // four device-coherent loads per lane cover 256 workgroups; a count is complete everywhere
+    // when every workgroup's progress word has reached it
     unsigned ready = 0, spins = 0;
     unsigned target = next_target(0u);
     const int rounds = (G + 255) >> 8;
+    const int masters = min(kMasters, G);
+    const bool master = b < masters;
+    unsigned *announce = g_announced + (b % masters) * kProgressStride;
     while (target) {
+      // nothing can be complete everywhere before it is complete here: stay off the memory system
+      // until this workgroup has reported the count in question
+      while (lds_load(&ctl->published) < target) __builtin_amdgcn_s_sleep(2);
       unsigned lo = 0xffffffffu;
-      for (int k = 0; k < rounds; ++k) {
-        const int first = (k * 64 + lane) * 4;
-        uint4_t v;
-        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
-                     : "=v"(v)
-                     : "v"(g_progress + first)
-                     : "memory");
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (first + i < G) lo = min(lo, v[i]);
+      if (!master) {
+        // the count announced by this workgroup's master
+        asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(lo) : "v"(announce) : "memory");
+      }
+      for (int k = 0; master && k < rounds; ++k) {
+        // (indices past the last workgroup read its word again)
+        const unsigned *p0 = g_progress + min(k * 256 + lane, G - 1) * kProgressStride;
+        const unsigned *p1 = g_progress + min(k * 256 + 64 + lane, G - 1) * kProgressStride;
+        const unsigned *p2 = g_progress + min(k * 256 + 128 + lane, G - 1) * kProgressStride;
+        const unsigned *p3 = g_progress + min(k * 256 + 192 + lane, G - 1) * kProgressStride;
+        unsigned v0, v1, v2, v3;
+        asm volatile(
+            "global_load_dword %0, %4, off sc1\n\t"
+            "global_load_dword %1, %5, off sc1\n\t"
+            "global_load_dword %2, %6, off sc1\n\t"
+            "global_load_dword %3, %7, off sc1\n\t"
+            "s_waitcnt vmcnt(0)"
+            : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
+            : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+            : "memory");
+        lo = min(min(lo, min(v0, v1)), min(v2, v3));
       }
       bool advanced = false;
       while (target && __builtin_amdgcn_ballot_w64(lo < target) == 0) {  // no lane below the target
@@ -235,7 +263,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         advanced = true;
       }
       if (advanced) {
-        if (lane == 0) __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lane == 0) {
+          __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (master) __hip_atomic_store(announce, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         spins = 0;
       } else if (++spins > kSpinLimit) {  // some workgroup is not running: give up, let everybody finish
         if (lane == 0) {
@@ -281,8 +312,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       }
       if (uni(cache[d].publish)) {
         wait_vm<0>();  // every lane's stores of this and of all earlier entries are complete ...
-        if (lane == 0)   // ... then publish
-          __hip_atomic_store(&g_progress[b], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) {  // ... then publish
+          __hip_atomic_store(&g_progress[b * kProgressStride], (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(&ctl->published, (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
       }
     }
     // a sequence without dependencies has not touched the progress words
@@ -294,7 +327,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     if (lane == 0) last = atomicAdd(&g_exited, 1u) == (unsigned)G - 1;
     if (uni((int)last)) {
       wait_vm<0>();
-      for (int i = lane; i < G; i += 64) __hip_atomic_store(&g_progress[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int i = lane; i < G; i += 64)
+        __hip_atomic_store(&g_progress[i * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane < kMasters)
+        __hip_atomic_store(&g_announced[lane * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     return;
