@@ -52,7 +52,7 @@ constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, 
 // announces the count that is complete everywhere in a word of its own, which the pollers of the
 // workgroups b with b % kMasters equal to its index watch (one more hop for a wait that is
 // exposed, 1/32 of the loads that collide with the stores).
-constexpr int kMaxGroups = 1024;
+constexpr int kMaxGroups = 256;  // (the watcher keeps a copy of every progress word in LDS)
 constexpr int kProgressStride = 32;  // words
 constexpr int kMasters = 1;
 __device__ __attribute__((aligned(128))) unsigned int g_progress[kMaxGroups * kProgressStride];
@@ -115,6 +115,14 @@ __device__ __forceinline__ unsigned lds_load(const unsigned *p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// LDS read the compiler does not see as such: after a direct-to-LDS load it makes every LDS read
+// that might alias wait for ALL outstanding loads
+__device__ __forceinline__ unsigned lds_peek(const unsigned *p) {
+  unsigned v;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"((uint32_t)(uintptr_t)p) : "memory");
+  return v;
+}
+
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ const char *uni_ptr(const void *p) {
   const uint64_t v = (uint64_t)(uintptr_t)p;
@@ -172,6 +180,8 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   // MC == 4 only: per wave, the group sums of the current x chunk, [half][kc][corr e0..3, xsum e0..3]
   // (registers are short in that variant)
   float *table = reinterpret_cast<float *>(ctl) + 16 + wave * 64;
+  // the watcher's copy of the progress words
+  unsigned *seen = reinterpret_cast<unsigned *>(ctl) + 16 + kWaves * 64;
 
   for (int i = tid; i < n_entries; i += kThreadsAll) {
     const Entry e = SINGLE ? single : entries[i];
@@ -192,6 +202,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     c.act = (char)e.activation;
     cache[i] = c;
   }
+  if (tid < kMaxGroups) seen[tid] = 0u;
   if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
   __syncthreads();
   // completion is reported only where an entry waits for it (a report costs the reducer a round
@@ -221,52 +232,57 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       }
       return 0u;
     };
-    // four device-coherent loads per lane cover 256 workgroups; a count is complete everywhere
-    // when every workgroup's progress word has reached it
+    // Reads of memory are direct-to-LDS loads that nobody waits for one by one: a new one is issued
+    // every ~100 ns with several in flight, so a change is seen one memory latency after it
+    // happened instead of up to two round trips later.  The values only grow, loads return in the
+    // order issued, so the LDS copies only grow too.
+    //   watcher: 4 loads copy the 256 progress words into `seen`; a count is complete everywhere
+    //            when every word has reached it; the result goes to ctl->ready and g_announced
+    //   others : one lane copies g_announced straight into ctl->ready, where the compute waves look
     unsigned ready = 0, spins = 0;
     unsigned target = next_target(0u);
-    const int rounds = (G + 255) >> 8;
-    const int masters = min(kMasters, G);
-    const bool master = b < masters;
-    unsigned *announce = g_announced + (b % masters) * kProgressStride;
+    const bool watcher = b == 0;
+    int lane_zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
     while (target) {
       // nothing can be complete everywhere before it is complete here: stay off the memory system
       // until this workgroup has reported the count in question
-      while (lds_load(&ctl->published) < target) __builtin_amdgcn_s_sleep(2);
-      unsigned lo = 0xffffffffu;
-      if (!master) {
-        // the count announced by this workgroup's master
-        asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(lo) : "v"(announce) : "memory");
-      }
-      for (int k = 0; master && k < rounds; ++k) {
-        // (indices past the last workgroup read its word again)
-        const unsigned *p0 = g_progress + min(k * 256 + lane, G - 1) * kProgressStride;
-        const unsigned *p1 = g_progress + min(k * 256 + 64 + lane, G - 1) * kProgressStride;
-        const unsigned *p2 = g_progress + min(k * 256 + 128 + lane, G - 1) * kProgressStride;
-        const unsigned *p3 = g_progress + min(k * 256 + 192 + lane, G - 1) * kProgressStride;
-        unsigned v0, v1, v2, v3;
-        asm volatile(
-            "global_load_dword %0, %4, off sc1\n\t"
-            "global_load_dword %1, %5, off sc1\n\t"
-            "global_load_dword %2, %6, off sc1\n\t"
-            "global_load_dword %3, %7, off sc1\n\t"
-            "s_waitcnt vmcnt(0)"
-            : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
-            : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
-            : "memory");
-        lo = min(min(lo, min(v0, v1)), min(v2, v3));
-      }
+      while (lds_peek(&ctl->published) < target) __builtin_amdgcn_s_sleep(2);
       bool advanced = false;
-      while (target && __builtin_amdgcn_ballot_w64(lo < target) == 0) {  // no lane below the target
-        ready = target;
-        target = next_target(ready);
-        advanced = true;
+      if (!watcher) {
+        // (the address must come from a vector register: with a uniform address the compiler
+        // emits a malformed instruction)
+        if (lane == 0)
+          __builtin_amdgcn_global_load_lds(g_announced + lane_zero, reinterpret_cast<unsigned *>(&ctl->ready), 4, 0,
+                                           kAuxDeviceCoherent);
+        wait_vm<7>();
+        __builtin_amdgcn_s_sleep(2);
+        const unsigned now = (unsigned)uni((int)lds_peek(&ctl->ready));
+        while (target && now >= target) {
+          ready = target;
+          target = next_target(ready);
+          advanced = true;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)  // (indices past the last workgroup read its word again)
+          __builtin_amdgcn_global_load_lds(g_progress + min(i * 64 + lane, G - 1) * kProgressStride, seen + i * 64, 4, 0,
+                                           kAuxDeviceCoherent);
+        wait_vm<8>();  // all but the two youngest sweeps have landed
+        __builtin_amdgcn_s_sleep(1);
+        unsigned lo = min(min(lds_peek(&seen[lane]), lds_peek(&seen[lane + 64])),
+                          min(lds_peek(&seen[lane + 128]), lds_peek(&seen[lane + 192])));
+        while (target && __builtin_amdgcn_ballot_w64(lo < target) == 0) {  // no lane below the target
+          ready = target;
+          target = next_target(ready);
+          advanced = true;
+        }
+        if (advanced && lane == 0) {
+          __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          __hip_atomic_store(g_announced, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
       if (advanced) {
-        if (lane == 0) {
-          __hip_atomic_store(&ctl->ready, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          if (master) __hip_atomic_store(announce, ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
         spins = 0;
       } else if (++spins > kSpinLimit) {  // some workgroup is not running: give up, let everybody finish
         if (lane == 0) {
@@ -276,6 +292,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         break;
       }
     }
+    wait_vm<0>();  // no load may land in LDS after this workgroup has gone
     return;
   }
 
@@ -724,7 +741,7 @@ int stream_grid(int *dev_out) {
 template <int MC, int NS>
 constexpr int stream_lds_bytes() {
   return kWaves * (NS * kItemBytes + kStageBytes) + kMaxEntries * 64 + 2 * kWaves * pass_rows(MC) * MC * 16 * 4 + 64 +
-         kWaves * 256;
+         kWaves * 256 + kMaxGroups * 4;
 }
 
 }  // namespace
