@@ -461,6 +461,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   const half_t *st_x = nullptr;  // the stage holds this wave's chunk of EVERY phase of (st_x, st_k, st_m)
   int st_k = 0, st_m = 0;
   unsigned known_ready = 0;  // entries this wave has seen complete on the whole device
+  // an entry whose x chunks do not fit the stage together fetches the chunk of its NEXT phase as
+  // soon as the operands of the current one are in registers, instead of draining the ring for it
+  int ahead_d = -1, ahead_chunk = -1;  // the stage holds (or will hold) this chunk of entry ahead_d
+  int ahead_after = 0;                 // items issued after that request (loads return in order)
 
   for (int d = 0; d < n_entries; ++d) {
     const int nrb = uni(cache[d].nrb), m_rows = uni(cache[d].m_rows), k_in = uni(cache[d].k_in);
@@ -501,13 +505,23 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         if (chunk * 512 >= k_in) continue;
         // ---- A operands and group sums of this chunk (kept when the previous entry used the same x)
         const bool reload_x = !(x_loaded == x && x_chunk == chunk && x_k == k_in && x_m == m_rows);
-        const bool drained = reload_x && !staged;
+        bool drained = false;
         if (reload_x) {
           if (!staged) {
-            for (int m = 0; m < m_rows; ++m)
-              __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
-                                               xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
-            wait_vm<0>();  // x is the youngest load: everything in flight lands with it
+            if (ahead_d == d && ahead_chunk == chunk) {
+              // requested ahead of time: older than the loads of ahead_after items
+              if (ahead_after >= 3) wait_vm<3 * kItemOps>();
+              else if (ahead_after == 2) wait_vm<2 * kItemOps>();
+              else if (ahead_after == 1) wait_vm<kItemOps>();
+              else wait_vm<0>();
+            } else {
+              for (int m = 0; m < m_rows; ++m)
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + lane,
+                                                 xstage + m * 1024, 16, 0, kAuxDeviceCoherent);
+              wait_vm<0>();  // x is the youngest load: everything in flight lands with it
+              drained = true;
+            }
+            ahead_d = -1;
             st_x = nullptr;
           }
           const uint32_t xs_rd = x_rd + (staged ? phase * m_rows * 1024 : 0);
@@ -575,6 +589,21 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           x_chunk = chunk;
           x_k = k_in;
           x_m = m_rows;
+          if (!staged && phases > 1) {
+            // the stage has been read: request this wave's chunk of the next phase (or of the first
+            // phase of the next pass) into it
+            int next_chunk = (phase + 1) * kWaves + wave;
+            if (phase + 1 >= phases || next_chunk * 512 >= k_in) next_chunk = (pass + 1) * PR < nrb ? wave : -1;
+            if (next_chunk >= 0 && next_chunk * 512 < k_in) {
+              for (int m = 0; m < m_rows; ++m)
+                __builtin_amdgcn_global_load_lds(
+                    reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + next_chunk * 512) + lane, xstage + m * 1024, 16,
+                    0, kAuxDeviceCoherent);
+              ahead_d = d;
+              ahead_chunk = next_chunk;
+              ahead_after = 0;
+            }
+          }
         }
 #pragma unroll
         for (int j = 0; j < PR; ++j) {
@@ -610,6 +639,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           if (prod.d < n_entries) {
             issue_item(prod, slot);
             ++n_ahead;
+            ++ahead_after;
             next_item(prod);
           }
           slot = slot + 1 == NS ? 0 : slot + 1;
