@@ -262,6 +262,17 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             seq.add(xs[ffn], *down[2:], ys[5], None, wait_for=b_)
             last = seq.add(xs[hidden], *o[2:], ys[3], None, wait_for=a)
 
+    def parallel_fused_qkv_ffn_first_streaming(seq):
+        # the same schedule with every weight in the streaming layout (gq_gemv_prepack_f16): the same
+        # bytes, stored as the contiguous 4608-byte blocks the kernel fetches
+        last = None
+        for layer in range(n_layers):
+            w_qkv, w_o, w_up, w_down = prepacked[layer]
+            b_ = seq.add(xs[hidden], w_up, None, None, ys[4], None, wait_for=last)
+            a = seq.add(xs[hidden], w_qkv, None, None, y_qkv, None)
+            seq.add(xs[ffn], w_down, None, None, ys[5], None, wait_for=b_)
+            last = seq.add(xs[hidden], w_o, None, None, ys[3], None, wait_for=a)
+
     def free(seq):
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
             seq.add(xs[k_in], p, s, b, ys[i % 6], None)
@@ -269,9 +280,12 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     fused_qkv = [tuple(torch.cat([mats[layer * 6 + role][2 + part] for role in range(3)], dim=0).contiguous()
                        for part in range(3)) for layer in range(n_layers)]
     y_qkv = torch.empty((m_rows, 3 * hidden), dtype=torch.float16, device=device)
+    prepacked = [(hip.prepack_gemv(*fused_qkv[layer]),) + tuple(hip.prepack_gemv(*mats[layer * 6 + role][2:]) for role in (3, 4, 5))
+                 for layer in range(n_layers)]
     for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
                        ("sequence_parallel_block_fused_qkv", parallel_fused_qkv),
                        ("sequence_parallel_block_fused_qkv_ffn_first", parallel_fused_qkv_ffn_first),
+                       ("sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", parallel_fused_qkv_ffn_first_streaming),
                        ("sequence_no_waits", free)):
         seq = hip.GemvSequence(device)
         fill(seq)

@@ -153,7 +153,8 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
  */
 typedef struct gq_gemv_desc {
   const uint16_t *x;        /* [m_rows, k_in] binary16 */
-  const uint16_t *packed;   /* [n_out, k_in / group_size, group_size / 4] */
+  const uint16_t *packed;   /* [n_out, k_in / group_size, group_size / 4]; or, with scale == bias == NULL,
+                               the weight in the streaming layout written by gq_gemv_prepack_f16 */
   const uint16_t *scale;    /* [n_out, k_in / group_size] binary16 */
   const uint16_t *bias;     /* [n_out, k_in / group_size] binary16 */
   const uint16_t *out_bias; /* [n_out] binary16 or NULL */
@@ -162,6 +163,26 @@ typedef struct gq_gemv_desc {
   int32_t wait_entries;     /* entries [0, wait_entries) complete before this one starts */
   int32_t activation;       /* GQ_ACT_*: epilogue of this entry */
 } gq_gemv_desc;
+
+/*
+ * Streaming layout of one weight for gq_gemv_sequence_f16.  No counterpart in the reference, whose
+ * three variables (popxl_addons/layers/linear_gq.py:74-97) stay what the rest of the API takes;
+ * this is a derived copy made once when the weights are loaded.  The persistent kernel fetches a
+ * weight in pieces of 16 rows x 512 input features: 4 KiB of packed words in sixteen 256-byte
+ * stretches one row apart, plus sixteen 16-byte pieces each of scale and bias.  The streaming
+ * layout stores every such piece as one contiguous 4608-byte block in the order the kernel keeps
+ * it in LDS (rows past n_out zero-filled), so that all of its loads are contiguous; the bytes per
+ * weight stay 0.5625.  Needs group_size 64 and k_in % 512 == 0.
+ *
+ *   gq_gemv_prepacked_bytes  size of the blob in bytes, or a negative GQ_ERR_* code
+ *   gq_gemv_prepack_f16      writes the blob (device memory, 16-byte aligned) from packed / scale /
+ *                            bias (16-byte aligned) on `stream`
+ * An entry of a sequence uses the blob by passing it as `packed` with scale == bias == NULL; such
+ * an entry needs m_rows <= 4 and a sequence that runs on the persistent kernel as a whole.
+ */
+int64_t gq_gemv_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size);
+int gq_gemv_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob,
+                        int64_t n_out, int64_t k_in, int64_t group_size, void *stream);
 
 int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
                          int32_t *status, void *stream);

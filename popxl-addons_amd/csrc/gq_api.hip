@@ -163,8 +163,21 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
     return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_f16: misaligned descs_device or status");
   for (int64_t i = 0; i < count; ++i) {
     const gq_gemv_desc &d = descs[i];
-    const int rc = gq::check_linear_args("gq_gemv_sequence_f16", d.x, d.m_rows, d.packed, d.scale, d.bias,
-                                         d.out_bias, d.y, d.n_out, d.k_in, d.group_size);
+    const bool blob = d.scale == nullptr && d.bias == nullptr && d.packed != nullptr;
+    if (blob) {
+      // the weight in the streaming layout: only the persistent kernel reads it
+      if (d.group_size != 64 || d.k_in <= 0 || d.k_in % 512 != 0 || d.m_rows < 1 || d.m_rows > 4 || d.n_out < 1)
+        return gq::fail(GQ_ERR_UNSUPPORTED,
+                        "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which needs group_size 64, "
+                        "k_in %% 512 == 0 and 1 <= m_rows <= 4 (got group_size=%d k_in=%d m_rows=%d n_out=%d)",
+                        (long long)i, d.group_size, d.k_in, d.m_rows, d.n_out);
+      if (gq::misaligned(d.packed, 16) || gq::misaligned(d.x, 16))
+        return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_f16: entry %lld: blob and x must be 16-byte aligned",
+                        (long long)i);
+    }
+    // (the blob stands in for scale and bias in the checks shared with the other entry points)
+    const int rc = gq::check_linear_args("gq_gemv_sequence_f16", d.x, d.m_rows, d.packed, blob ? d.packed : d.scale,
+                                         blob ? d.packed : d.bias, d.out_bias, d.y, d.n_out, d.k_in, d.group_size);
     if (rc < 0) return rc;
     if (rc == 0 || d.k_in == 0)
       return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld is empty", (long long)i);
@@ -179,6 +192,28 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
                       (long long)i, d.wait_entries, (long long)i);
   }
   return gq::launch_gemv_sequence(descs, descs_device, count, status, (hipStream_t)stream);
+}
+
+int64_t gq_gemv_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (n_out < 0 || k_in < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_prepacked_bytes: negative size");
+  if (group_size != 64 || k_in % 512 != 0)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_prepacked_bytes: the streaming layout needs group_size 64 and k_in %% 512 == 0 "
+                                        "(got group_size=%lld k_in=%lld)", (long long)group_size, (long long)k_in);
+  if (n_out > (1 << 22) || k_in > (1 << 24))
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_prepacked_bytes: n_out=%lld or k_in=%lld too large", (long long)n_out,
+                    (long long)k_in);
+  return gq::gemv_prepacked_bytes(n_out, k_in);
+}
+
+int gq_gemv_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
+                        int64_t k_in, int64_t group_size, void *stream) {
+  const int64_t bytes = gq_gemv_prepacked_bytes(n_out, k_in, group_size);
+  if (bytes < 0) return (int)bytes;
+  if (bytes == 0) return GQ_OK;
+  if (!packed || !scale || !bias || !blob) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_prepack_f16: NULL pointer argument");
+  if (gq::misaligned(packed, 16) || gq::misaligned(scale, 16) || gq::misaligned(bias, 16) || gq::misaligned(blob, 16))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_prepack_f16: pointers must be 16-byte aligned");
+  return gq::launch_gemv_prepack(packed, scale, bias, blob, n_out, k_in, (hipStream_t)stream);
 }
 
 int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,

@@ -52,6 +52,9 @@ int launch_gemv_streamed(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                          int64_t group_size, int act, hipStream_t stream);
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
                          hipStream_t stream);
+int64_t gemv_prepacked_bytes(int64_t n_out, int64_t k_in);
+int launch_gemv_prepack(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
+                        int64_t k_in, hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
                     int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
 

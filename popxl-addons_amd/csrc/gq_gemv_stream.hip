@@ -11,6 +11,10 @@
 //   row block  = 16 weight rows; workgroup b of G owns row blocks b, b + G, ... in passes of 4 (2 when MC = 4)
 //   phase      = 4096 contraction indices; wave w owns chunk 8 p + w (512 indices) of phase p
 //   work item  = (row block, chunk): 4 KiB of packed words + 2 x 256 B of scale / bias
+// An entry may bring its weight in the streaming layout instead (scale == bias == nullptr, made by
+// gq_gemv_prepack_f16): work item (row block rb, chunk c) is the 4608-byte block number
+// rb * (k_in / 512) + c, byte for byte what the item's ring slot holds, so that its loads are
+// 1 KiB contiguous each instead of sixteen 64-byte or 16-byte pieces 128+ bytes apart.
 //
 // Arithmetic.  Once the weights stream without gaps the loop is bound by instruction issue, not by
 // HBM, so the expansion of the codes is kept to 5 VALU instructions per 8 weights: a code is only
@@ -363,7 +367,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   struct ProducerEntry {
     const char *packed, *scale, *bias;
     int n_out, k_in, nrb, phases;
-  } pe = {nullptr, nullptr, nullptr, 1, 512, 0, 1};
+  } pe = {nullptr, nullptr, nullptr, 1, 512, 0, 1};  // (scale == nullptr: streaming layout)
   auto load_producer_entry = [&](int d) {
     if (d >= n_entries) return;
     pe.packed = uni_ptr(cache[d].packed);
@@ -401,6 +405,16 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     const int chunk = c.phase * kWaves + wave;
     const int row = min(r, pe.n_out - 1 - rb * 16);  // rows past n_out re-read the last one
     char *dst = ring + slot * kItemBytes;
+    if (pe.scale == nullptr) {
+      const char *blk = pe.packed + ((int64_t)rb * (pe.k_in >> 9) + chunk) * kItemBytes + lane * 16;
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + s * 1024), dst + s * 1024, 16, 0, 0);
+      // (two loads of 256 bytes, like the other layout: every item counts kItemOps loads)
+      if (kc == 0) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, 0);
+      if (kc == 1) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, 0);
+      return;
+    }
     const char *src = pe.packed + (int64_t)rb * 16 * (pe.k_in >> 1) + chunk * 256;
     const uint32_t off = (uint32_t)row * (uint32_t)(pe.k_in >> 1) + (uint32_t)kc * 16u;
 #pragma unroll
@@ -743,6 +757,8 @@ __global__ __launch_bounds__(kThreadsAll) void gemv_stream_single_kernel(const g
 
 namespace {
 
+bool prepacked(const gq_gemv_desc &d) { return d.scale == nullptr && d.bias == nullptr; }
+
 bool stream_shape_ok(const gq_gemv_desc &d) {
   return d.group_size == 64 && d.k_in % 512 == 0 && d.k_in > 0 && d.k_in <= (1 << 24) && d.m_rows >= 1 &&
          d.m_rows <= 4 && d.n_out >= 1 && d.n_out <= (1 << 22) && ((uintptr_t)d.x % 16) == 0 &&
@@ -829,6 +845,12 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   }
   if (!supported || option_gemv_variant() == 3) {
     // any other shape: one launch per entry; stream order provides every dependency
+    for (int64_t i = 0; i < count; ++i)
+      if (prepacked(host[i]))
+        return fail(GQ_ERR_UNSUPPORTED,
+                    "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which only the persistent kernel "
+                    "reads, but the sequence holds a shape outside it (group 64, k_in %% 512 == 0, m_rows <= 4, 16-byte "
+                    "aligned)", (long long)i);
     for (int64_t i = 0; i < count; ++i) {
       const gq_gemv_desc &d = host[i];
       const int rc = launch_gemv(d.x, d.m_rows, d.packed, d.scale, d.bias, d.out_bias, d.y, d.n_out, d.k_in,
@@ -861,6 +883,49 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   else GQ_STREAM(4, 3);
 #undef GQ_STREAM
   return check_launch("gemv_stream_kernel");
+}
+
+// ---- the streaming layout: block (rb, c) = what the ring slot of work item (rb, c) holds
+namespace {
+
+__global__ __launch_bounds__(256) void prepack_kernel(const char *__restrict__ packed, const char *__restrict__ scale,
+                                                      const char *__restrict__ bias, uint4_t *__restrict__ blob, int n_out,
+                                                      int k_in, int64_t units) {
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;  // 16-byte unit of the blob
+  if (u >= units) return;
+  constexpr int kUnits = kItemBytes / 16;
+  const int64_t block = u / kUnits;
+  const int w = (int)(u % kUnits), chunks = k_in >> 9;
+  const int64_t rb = block / chunks;
+  const int c = (int)(block % chunks);
+  const int r = w & 15;
+  const int64_t row = rb * 16 + r;
+  uint4_t v = {0u, 0u, 0u, 0u};  // rows past n_out: code 0, scale 0, bias 0
+  if (row < n_out) {
+    if (w < 256) {
+      const int s = w >> 6, kc = (w >> 4) & 3;  // slot layout [s][kc][r]: bytes s * 64 + kc * 16 of the row's chunk
+      v = *reinterpret_cast<const uint4_t *>(packed + row * (k_in >> 1) + c * 256 + s * 64 + kc * 16);
+    } else {
+      const char *src = w < 272 ? scale : bias;  // the 8 values of the row's chunk
+      v = *reinterpret_cast<const uint4_t *>(src + row * (k_in >> 5) + c * 16);
+    }
+  }
+  blob[u] = v;
+}
+
+}  // namespace
+
+int64_t gemv_prepacked_bytes(int64_t n_out, int64_t k_in) { return ((n_out + 15) / 16) * (k_in / 512) * kItemBytes; }
+
+int launch_gemv_prepack(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
+                        int64_t k_in, hipStream_t stream) {
+  const int64_t units = gemv_prepacked_bytes(n_out, k_in) / 16;
+  const int64_t blocks = (units + 255) / 256;
+  if (blocks > 0x7fffffff) return fail(GQ_ERR_UNSUPPORTED, "gq_gemv_prepack_f16: weight too large");
+  prepack_kernel<<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      reinterpret_cast<const char *>(packed), reinterpret_cast<const char *>(scale), reinterpret_cast<const char *>(bias),
+      reinterpret_cast<uint4_t *>(blob), (int)n_out, (int)k_in, units);
+  return check_launch("prepack_kernel");
 }
 
 }  // namespace gq

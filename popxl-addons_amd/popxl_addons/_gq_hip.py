@@ -41,6 +41,8 @@ EXPORTS = (
     "gq_linear_f16",
     "gq_linear_act_f16",
     "gq_gemv_sequence_f16",
+    "gq_gemv_prepacked_bytes",
+    "gq_gemv_prepack_f16",
     "gq_compress_f16",
 )
 
@@ -92,6 +94,10 @@ def load():
     lib.gq_linear_act_f16.restype = ctypes.c_int
     lib.gq_gemv_sequence_f16.argtypes = [p, p, i64, p, p]
     lib.gq_gemv_sequence_f16.restype = ctypes.c_int
+    lib.gq_gemv_prepacked_bytes.argtypes = [i64, i64, i64]
+    lib.gq_gemv_prepacked_bytes.restype = i64
+    lib.gq_gemv_prepack_f16.argtypes = [p, p, p, p, i64, i64, i64, p]
+    lib.gq_gemv_prepack_f16.restype = ctypes.c_int
     lib.gq_compress_f16.argtypes = [p, p, p, p, p, i64, i64, i64, p]
     lib.gq_compress_f16.restype = ctypes.c_int
     if lib.gq_abi_version() != GQ_ABI_VERSION:
@@ -114,6 +120,33 @@ def call(name, *args):
 
 def set_option(name, value):
     call("gq_set_option", name.encode(), int(value))
+
+
+class PrepackedWeight:
+    """One weight in the streaming layout of gq_gemv_prepack_f16 (a device blob that only
+    GemvSequence entries read); made from the three LinearGQ variables by prepack_gemv()."""
+
+    def __init__(self, blob, n_out, k_in, group_size):
+        self.blob, self.n_out, self.k_in, self.group_size = blob, n_out, k_in, group_size
+
+
+def prepack_gemv(packed, scale, bias):
+    """packed uint16 [n_out, G, I], scale / bias float16 [n_out, G, 1] on the GPU -> PrepackedWeight."""
+    import torch
+
+    n_out, n_groups, n_ids = packed.shape
+    k_in, group_size = n_groups * n_ids * 4, n_ids * 4
+    for t in (packed, scale, bias):
+        assert t.is_cuda and t.is_contiguous()
+    lib = load()
+    nbytes = lib.gq_gemv_prepacked_bytes(n_out, k_in, group_size)
+    if nbytes < 0:
+        raise GQHipError("gq_gemv_prepacked_bytes", nbytes, lib.gq_last_error().decode("utf-8", "replace"))
+    with torch.cuda.device(packed.device):
+        blob = torch.empty(nbytes, dtype=torch.uint8, device=packed.device)
+        call("gq_gemv_prepack_f16", packed.data_ptr(), scale.data_ptr(), bias.data_ptr(), blob.data_ptr(), n_out, k_in,
+             group_size, torch.cuda.current_stream(packed.device).cuda_stream)
+    return PrepackedWeight(blob, n_out, k_in, group_size)
 
 
 class GemvSequence:
@@ -143,18 +176,29 @@ class GemvSequence:
         self.status = None
 
     def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None, activation=None):
+        """`packed` may be a PrepackedWeight (then scale and bias are None)."""
         m_rows, k_in = x.shape
-        n_out, n_groups, n_ids = packed.shape
-        assert y.shape == (m_rows, n_out) and n_groups * n_ids * 4 == k_in
-        for t in (x, packed, scale, bias, y):
+        if isinstance(packed, PrepackedWeight):
+            assert scale is None and bias is None and packed.k_in == k_in
+            n_out, group_size = packed.n_out, packed.group_size
+            pointers = (packed.blob.data_ptr(), 0, 0)
+            tensors = (x, packed.blob, y)
+        else:
+            n_out, n_groups, n_ids = packed.shape
+            assert n_groups * n_ids * 4 == k_in
+            group_size = n_ids * 4
+            pointers = (packed.data_ptr(), scale.data_ptr(), bias.data_ptr())
+            tensors = (x, packed, scale, bias, y)
+        assert y.shape == (m_rows, n_out)
+        for t in tensors:
             assert t.is_cuda and t.is_contiguous()
         index = len(self.entries)
         wait_entries = index if wait_previous else (0 if wait_for is None else int(wait_for) + 1)
         if not 0 <= wait_entries <= index:
             raise ValueError(f"entry {index} cannot wait for entry {wait_for}")
         self.entries.append(
-            (x.data_ptr(), packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
-             0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, n_ids * 4,
+            (x.data_ptr(), *pointers,
+             0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, group_size,
              wait_entries, activation_code(activation))
         )
         self.keep.append((x, packed, scale, bias, y, out_bias))

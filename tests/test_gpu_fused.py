@@ -222,6 +222,55 @@ def test_gemv_sequence_chained_entries(hip, device, oracle, m_rows):
             x_prev = yy
 
 
+@pytest.mark.parametrize("m_rows,chained", [(1, False), (2, False), (4, False), (1, True), (4, True)])
+def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
+    """Weights in the streaming layout of gq_gemv_prepack_f16 give bit for bit what the same
+    sequence gives on the three variables (same arithmetic, other addresses), with ragged row
+    counts, waits, and both layouts mixed in one sequence."""
+    from popxl_addons._gq_hip import GemvSequence, GQHipError, prepack_gemv
+
+    if chained:
+        shapes = [(4096, 4096), (2048, 4096), (4096, 2048), (16384, 4096), (4096, 16384), (520, 4096)]
+    else:
+        shapes = [(4096, 4096), (1000, 4096), (16384, 4096), (4096, 16384), (16, 512), (5000, 1536), (40, 8192)]
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, m_rows, chained=chained)
+    for mixed in (False, True):
+        seq2, outs2 = GemvSequence(device), []
+        for i, (x, packed, scale, bias, y, ob) in enumerate(seq.keep):
+            y2 = torch.full_like(y, float("nan"))
+            x2 = outs2[-1] if chained and i > 0 else x
+            if mixed and i % 3 == 1:
+                seq2.add(x2, packed, scale, bias, y2, ob, wait_previous=chained and i > 0)
+            else:
+                w = prepack_gemv(packed, scale, bias)
+                assert w.blob.numel() == int(-(-packed.shape[0] // 16) * 16 * x.shape[1] * 0.5625)
+                seq2.add(x2, w, None, None, y2, ob, wait_previous=chained and i > 0)
+            outs2.append(y2)
+        for _ in range(2):
+            for y in outs + outs2:
+                y.fill_(float("nan"))
+            seq.run()
+            seq2.run()
+            torch.cuda.synchronize()
+            assert int(seq.status.item()) == 0 and int(seq2.status.item()) == 0
+            for i, (y, y2) in enumerate(zip(outs, outs2)):
+                assert torch.isfinite(y2).all(), i
+                assert torch.equal(y, y2), (i, mixed)
+        if not chained:
+            for y2, ref in zip(outs2, refs):
+                assert normalised_error(y2.cpu().numpy(), ref) <= TOL
+    # a blob next to an entry that only the per-entry kernels can run (group 32) is refused
+    rng = np.random.default_rng(4)
+    p32, s32, b32 = (to_dev(a, device) for a in group_quantize_compress_numpy(rng.normal(0, 0.02, (96, 256)).astype(np.float16), 32))
+    bad = GemvSequence(device)
+    x, packed, scale, bias, y, ob = seq.keep[0]
+    bad.add(x, prepack_gemv(packed, scale, bias), None, None, y, ob)
+    bad.add(to_dev(activations(m_rows, 256, 1), device), p32, s32, b32, torch.empty((m_rows, 96), dtype=torch.float16, device=device))
+    with pytest.raises(GQHipError) as e:
+        bad.run()
+    assert "streaming layout" in str(e.value)
+
+
 def test_gemv_sequence_fallback_and_graph(hip, device, oracle):
     """Shapes outside the persistent kernel (group 32) run entry by entry; the persistent kernel
     replays correctly from a captured graph."""

@@ -77,6 +77,34 @@ def test_abi_version_and_error_text_without_gpu():
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
     assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "activation" in str(e.value)
+    # the streaming layout: its size, what it needs, and what an entry that uses it needs
+    lib = _gq_hip.load()
+    assert lib.gq_gemv_prepacked_bytes(4096, 4096, 64) == 256 * 8 * 4608 == int(4096 * 4096 * 0.5625)
+    assert lib.gq_gemv_prepacked_bytes(1000, 1536, 64) == 63 * 3 * 4608  # rows padded to 16
+    assert lib.gq_gemv_prepacked_bytes(0, 512, 64) == 0
+    assert lib.gq_gemv_prepacked_bytes(64, 512, 32) == _gq_hip.GQ_ERR_UNSUPPORTED
+    assert lib.gq_gemv_prepacked_bytes(64, 448, 64) == _gq_hip.GQ_ERR_UNSUPPORTED and "512" in _gq_hip.last_error()
+    assert lib.gq_gemv_prepacked_bytes(-1, 512, 64) == _gq_hip.GQ_ERR_BAD_SHAPE
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_prepack_f16", 16, 16, 16, 0, 64, 512, 64, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_prepack_f16", 16, 16, 8, 16, 64, 512, 64, None)
+    assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED
+    desc["ptrs"] = [[16, 16, 16, 16, 0, 16], [16, 16, 0, 0, 0, 16]]  # entry 1: scale == bias == NULL
+    desc["ints"] = [[1, 8, 512, 64, 0, 0], [5, 8, 512, 64, 1, 0]]
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "streaming layout" in str(e.value)
+    desc["ints"] = [[1, 8, 512, 64, 0, 0], [1, 8, 512, 32, 1, 0]]
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "streaming layout" in str(e.value)
+    desc["ptrs"] = [[16, 16, 16, 16, 0, 16], [16, 16, 0, 16, 0, 16]]  # only scale NULL: not a blob, an error
+    desc["ints"] = [[1, 8, 512, 64, 0, 0], [1, 8, 512, 64, 1, 0]]
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
     assert _gq_hip.activation_code("gelu_tanh") == _gq_hip.GQ_ACT_GELU_TANH and _gq_hip.activation_code(None) == 0
     with pytest.raises(ValueError):
         _gq_hip.activation_code("swish")
