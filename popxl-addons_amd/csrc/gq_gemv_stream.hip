@@ -246,6 +246,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     unsigned ready = 0, spins = 0;
     unsigned target = next_target(0u);
     const bool watcher = b == 0;
+    unsigned last_seen[4] = {0u, 0u, 0u, 0u};  // watcher: this lane's four progress words as last read
     int lane_zero;
     asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
     while (target) {
@@ -268,14 +269,18 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
           advanced = true;
         }
       } else {
+        // only the words that have not reached the target yet: once most workgroups are through,
+        // a sweep is a handful of loads, and the watcher's own compute unit keeps its bandwidth
 #pragma unroll
         for (int i = 0; i < 4; ++i)  // (indices past the last workgroup read its word again)
-          __builtin_amdgcn_global_load_lds(g_progress + min(i * 64 + lane, G - 1) * kProgressStride, seen + i * 64, 4, 0,
-                                           kAuxDeviceCoherent);
-        wait_vm<8>();  // all but the two youngest sweeps have landed
+          if (last_seen[i] < target)
+            __builtin_amdgcn_global_load_lds(g_progress + min(i * 64 + lane, G - 1) * kProgressStride, seen + i * 64, 4, 0,
+                                             kAuxDeviceCoherent);
+        wait_vm<8>();  // bounds the loads in flight (a sweep is at most 4)
         __builtin_amdgcn_s_sleep(1);
-        unsigned lo = min(min(lds_peek(&seen[lane]), lds_peek(&seen[lane + 64])),
-                          min(lds_peek(&seen[lane + 128]), lds_peek(&seen[lane + 192])));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) last_seen[i] = lds_peek(&seen[i * 64 + lane]);
+        unsigned lo = min(min(last_seen[0], last_seen[1]), min(last_seen[2], last_seen[3]));
         while (target && __builtin_amdgcn_ballot_w64(lo < target) == 0) {  // no lane below the target
           ready = target;
           target = next_target(ready);
