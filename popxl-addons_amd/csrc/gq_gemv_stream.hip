@@ -544,7 +544,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             st_x = nullptr;
           }
           const uint32_t xs_rd = x_rd + (staged ? phase * m_rows * 1024 : 0);
+          // a lane whose slice lies outside its group, or whose batch row does not exist, supplies
+          // zeros: it keeps no operand (my_load matches no step) and its sums are dropped
           const bool active = a_match && a_m < m_rows;
+          const int my_load = active ? a_load : -1;
           constexpr int HALVES = MC == 2 ? 1 : 2;
           float part_sum[HALVES], part_corr[HALVES];
 #pragma unroll
@@ -561,7 +564,6 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             float s1 = 0.f, s2 = 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              if (!active) xq[j] = uint4_t{0u, 0u, 0u, 0u};  // rows of x that were not loaded may hold anything
 #pragma unroll
               for (int t = 0; t < 4; ++t) {
                 s1 = __builtin_amdgcn_fdot2(as_half2(xq[j][t]), kOnes, s1, false);
@@ -570,12 +572,13 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
               const half8_t p = permute_x(xq[j]);
               if (MC == 2) {
 #pragma unroll
-                for (int L = 0; L < 4; ++L) xa[L][j] = a_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                for (int L = 0; L < 4; ++L) xa[L][j] = my_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
               } else {
 #pragma unroll
-                for (int L = 0; L < 2; ++L) xa[L + 2 * h][j] = a_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                for (int L = 0; L < 2; ++L) xa[L + 2 * h][j] = my_load == L ? p : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
               }
             }
+            if (!active) s1 = s2 = 0.f;  // (rows of x that were not loaded may hold anything)
             // the other half of the group sits in the neighbouring slice
             part_sum[h] = s1 + lane_read(s1, lane ^ 16);
             part_corr[h] = s2 + lane_read(s2, lane ^ 16);
