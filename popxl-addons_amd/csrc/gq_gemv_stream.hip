@@ -52,15 +52,14 @@ constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, 
 // store hit a line that all 256 pollers were reading, and the stream of weights lost 4 - 5 us per
 // published entry (measured: polling lines that nobody writes, or writing lines that nobody
 // polls, costs nothing).
-// For the same reason only the pollers of the first kMasters workgroups read those words; each
-// announces the count that is complete everywhere in a word of its own, which the pollers of the
-// workgroups b with b % kMasters equal to its index watch (one more hop for a wait that is
-// exposed, 1/32 of the loads that collide with the stores).
+// For the same reason only ONE poller, the watcher (workgroup 0), reads those words; it announces
+// the count that is complete everywhere in a word of its own, which all other pollers watch (one
+// more hop for a wait that is exposed; measured: one watcher beats eight, and a watcher workgroup
+// without rows of its own loses more to the uneven split of the row blocks than it gains).
 constexpr int kMaxGroups = 256;  // (the watcher keeps a copy of every progress word in LDS)
 constexpr int kProgressStride = 32;  // words
-constexpr int kMasters = 1;
 __device__ __attribute__((aligned(128))) unsigned int g_progress[kMaxGroups * kProgressStride];
-__device__ __attribute__((aligned(128))) unsigned int g_announced[kMasters * kProgressStride];
+__device__ __attribute__((aligned(128))) unsigned int g_announced[kProgressStride];
 __device__ unsigned int g_exited;  // workgroups that left the kernel
 
 struct Entry {  // = gq_gemv_desc
@@ -158,9 +157,12 @@ __device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint3
 // wave drops its 16 x m partial sums into its mailbox (two sets, used by passes in turn, so a wave
 // may run a pass ahead of the slowest) and goes on with the next pass or entry.
 // Wave 8, the reducer, adds the eight mailboxes in a fixed order, stores y and, for entries that
-// somebody waits for, publishes the workgroup's progress.  Wave 9, the poller, watches the
-// progress words of all workgroups and publishes in LDS how many entries are complete everywhere;
-// a compute wave that needs an earlier result waits for that number only.
+// somebody waits for, publishes the workgroup's progress.  Wave 9, the poller, keeps the LDS word
+// `ready` (how many entries are complete everywhere) up to date: the watcher's from the progress
+// words of all workgroups, everybody else's from the watcher's announcement; a compute wave that
+// needs an earlier result waits for that number only.  (The LDS reads of `ready` and `consumed`
+// in the compute waves are visible to the compiler, which therefore waits for all loads of the
+// ring before them; hiding them in assembly was measured and gains nothing.)
 //
 // Visibility of results between compute units needs no cache flush: y is written with device-scope
 // stores (sc1, write-through to the coherent level), the reducer waits for its stores before it
@@ -355,8 +357,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       wait_vm<0>();
       for (int i = lane; i < G; i += 64)
         __hip_atomic_store(&g_progress[i * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (lane < kMasters)
-        __hip_atomic_store(&g_announced[lane * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(g_announced, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     return;
