@@ -217,13 +217,19 @@ __device__ __forceinline__ void wait_lds(uint4_t &a) {
 // ---------------------------------------------------------------------------------------
 constexpr int kWStages = 3;
 
-template <int WM, int WN, int FM, int FN, int XS>
+// KS: groups of WM x WN waves that split the contraction between them (group g takes the g-th
+// part of the K tiles, with an x ring of its own) and add their accumulators through LDS at the
+// end.  For small batches, where a workgroup per compute unit with one wave per SIMD leaves every
+// latency of the K step exposed: twice the waves on the same output tile, no more weight expansion.
+template <int WM, int WN, int FM, int FN, int XS, int KS = 1>
 struct Pipe2Shape {
   static constexpr int NW = WM * WN, TM = 32 * FM, TN = 32 * FN, TILE_M = WM * TM, TILE_N = WN * TN;
   static constexpr int X_STAGE = TILE_M * 128, W_STAGE = FN * 1280;
-  static constexpr int X_BYTES = XS * X_STAGE, LDS_BYTES = X_BYTES + NW * kWStages * W_STAGE;
+  static constexpr int X_BYTES = XS * X_STAGE, LDS_BYTES = KS * (X_BYTES + NW * kWStages * W_STAGE);
   static constexpr int A_OPS = TILE_M / 8 / NW;
   static constexpr int OPS = A_OPS + 3 * FN;
+  static constexpr int REDUCE_BYTES = (KS - 1) * NW * FM * FN * 16 * 256;  // accumulators of groups 1.. as floats
+  static_assert(REDUCE_BYTES <= LDS_BYTES, "the accumulators of the other groups must fit the rings");
 };
 
 // The 16 VALU instructions that turn one packed word into a B operand, cut into PIECES slices so
@@ -257,33 +263,36 @@ __device__ __forceinline__ half8_t dequant_result(const DequantState &st) {
                                  __builtin_shufflevector(st.w[2], st.w[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <int WM, int WN, int FM, int FN, int XS>
+template <int WM, int WN, int FM, int FN, int XS, int KS>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
     int gs_shift, int act) {
-  using S = Pipe2Shape<WM, WN, FM, FN, XS>;
+  using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
   constexpr int NW = S::NW, TM = S::TM, TN = S::TN, TILE_M = S::TILE_M, TILE_N = S::TILE_N;
   constexpr int A_OPS = S::A_OPS, OPS = S::OPS;
   static_assert(TILE_M % (8 * NW) == 0, "x tile must split evenly over the waves");
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // `wave` is the wave's index within its group of NW; the group takes K tiles [tile0, tile0 + n_tiles)
+  const int tid = threadIdx.x, lane = tid & 63, kgrp = (tid >> 6) / NW, wave = (tid >> 6) % NW;
   const int wm = wave / WN, wn = wave % WN;
   const int m0 = blockIdx.y * TILE_M, n0 = blockIdx.x * TILE_N;
   const int groups_per_row = k_in >> gs_shift;
-  const int n_tiles = k_in >> 6;
+  const int n_tiles = (k_in >> 6) / KS;  // (the launcher checks divisibility)
+  const int tile0 = kgrp * n_tiles;
 
   const half_t *a_src[A_OPS];
 #pragma unroll
   for (int q = 0; q < A_OPS; ++q) {
     const int slot = (q * NW + wave) * 64 + lane;
     const int r = slot >> 3, c = (slot & 7) ^ ((r >> 1) & 7);
-    a_src[q] = x + (int64_t)min(m0 + r, m_rows - 1) * k_in + c * 8;
+    a_src[q] = x + (int64_t)min(m0 + r, m_rows - 1) * k_in + c * 8 + tile0 * 64;
   }
   const int fr = lane & 31, h = lane >> 5;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const uint32_t a_rd_row = lds_base + (wm * TM + fr) * 128;
+  char *x_ring = lds + kgrp * S::X_BYTES;
+  const uint32_t a_rd_row = lds_base + kgrp * S::X_BYTES + (wm * TM + fr) * 128;
   uint32_t a_rd_chunk[4];
 #pragma unroll
   for (int s4 = 0; s4 < 4; ++s4) a_rd_chunk[s4] = ((4 * h + s4) ^ ((lane >> 1) & 7)) * 16;
@@ -293,21 +302,21 @@ __device__ __forceinline__ void gemm_pipe2_body(
 #pragma unroll
   for (int f = 0; f < FN; ++f) {
     const int row = min(n0 + wn * TN + f * 32 + fr, n_out - 1);
-    b_src[f] = packed + (int64_t)row * (k_in >> 5) + h;
+    b_src[f] = packed + (int64_t)row * (k_in >> 5) + h + tile0 * 2;
     s_src[f] = reinterpret_cast<const uint32_t *>(scale + (int64_t)row * groups_per_row);
     z_src[f] = reinterpret_cast<const uint32_t *>(bias + (int64_t)row * groups_per_row);
   }
-  char *w_ring = lds + S::X_BYTES + wave * (kWStages * S::W_STAGE);
-  const uint32_t w_rd = lds_base + S::X_BYTES + wave * (kWStages * S::W_STAGE);
+  char *w_ring = lds + KS * S::X_BYTES + (kgrp * NW + wave) * (kWStages * S::W_STAGE);
+  const uint32_t w_rd = lds_base + KS * S::X_BYTES + (kgrp * NW + wave) * (kWStages * S::W_STAGE);
 
   // Direct-to-LDS load number `op` (0 .. OPS-1) of tile `t_load` into the ring slots of tile number
   // `t_slot`: A_OPS chunks of the x tile, FN packed fragments, FN scale and FN bias dwords.
   // The two lanes (n, 0) and (n, 1) share one dword of scale and of bias (their groups are the
   // same, or the two halves of it): lanes with h == 0 fetch it.
   auto issue_op = [&](int op, int t_load, int t_slot) {
-    char *xs = lds + (t_slot % XS) * S::X_STAGE;
+    char *xs = x_ring + (t_slot % XS) * S::X_STAGE;
     char *ws = w_ring + (t_slot % kWStages) * S::W_STAGE;
-    const int g = (t_load * 64 + h * 32) >> gs_shift;
+    const int g = ((tile0 + t_load) * 64 + h * 32) >> gs_shift;
 #pragma unroll
     for (int q = 0; q < A_OPS; ++q)
       if (op == q) __builtin_amdgcn_global_load_lds(a_src[q] + t_load * 64, xs + (q * NW + wave) * 1024, 16, 0, 0);
@@ -335,7 +344,7 @@ __device__ __forceinline__ void gemm_pipe2_body(
     }
   };
   auto half_select = [&](int t) -> uint32_t {
-    const int g = (t * 64 + h * 32) >> gs_shift;
+    const int g = ((tile0 + t) * 64 + h * 32) >> gs_shift;
     return (g & 1) ? 0x07060706u : 0x05040504u;
   };
 
@@ -460,6 +469,33 @@ __device__ __forceinline__ void gemm_pipe2_body(
   wait_vmcnt<0>();  // surplus prefetches past the last tile
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
+  if (KS > 1) {
+    // the groups' partial sums meet in LDS (over the rings, which nobody reads any more):
+    // [group - 1][wave][accumulator][element][lane], group 0 adds them to its own
+    float *red = reinterpret_cast<float *>(lds);
+    __builtin_amdgcn_s_barrier();
+    if (kgrp > 0) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int f = 0; f < FN; ++f)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            red[((((kgrp - 1) * NW + wave) * FM * FN + i * FN + f) * 16 + e) * 64 + lane] = acc[i][f][e];
+    }
+    __builtin_amdgcn_s_barrier();
+    if (kgrp > 0) return;
+#pragma unroll
+    for (int g = 1; g < KS; ++g)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int f = 0; f < FN; ++f)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            acc[i][f][e] += red[((((g - 1) * NW + wave) * FM * FN + i * FN + f) * 16 + e) * 64 + lane];
+  }
+
   // D[m][n]: lane holds n = lane % 32 and m = 8 * (e / 4) + 4 * (lane / 32) + e % 4
   const bool interior = m0 + TILE_M <= m_rows && n0 + TILE_N <= n_out;
 #pragma unroll
@@ -490,24 +526,24 @@ __device__ __forceinline__ void gemm_pipe2_body(
 
 // (external linkage: their address is taken on the host for hipFuncSetAttribute)
 // OCC: waves per SIMD the register budget is sized for (2: 256 registers per lane, 1: 512)
-template <int WM, int WN, int FM, int FN, int XS, int OCC>
-__global__ __launch_bounds__(WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
+template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS>
+__global__ __launch_bounds__(KS * WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
                                                                   const half_t *scale, const half_t *bias,
                                                                   const half_t *out_bias, half_t *y, int n_out,
                                                                   int k_in, int gs_shift, int act) {
-  gemm_pipe2_body<WM, WN, FM, FN, XS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act);
+  gemm_pipe2_body<WM, WN, FM, FN, XS, KS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act);
 }
 
 namespace {
 
-template <int WM, int WN, int FM, int FN, int XS, int OCC>
+template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS = 1>
 int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int gs_shift,
                  int act, hipStream_t stream) {
-  using S = Pipe2Shape<WM, WN, FM, FN, XS>;
+  using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
   constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
   static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
-  auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC>;
+  auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC, KS>;
   // the attribute belongs to the (function, device) pair; same value every time: a benign race
   constexpr int kMaxDevices = 64;
   static bool configured[kMaxDevices] = {false};
@@ -521,7 +557,7 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
   }
   const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M));
   if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_gemm_f16: m_rows=%lld too large", (long long)m_rows);
-  kern<<<grid, dim3(WM * WN * 64), lds_bytes, stream>>>(
+  kern<<<grid, dim3(KS * WM * WN * 64), lds_bytes, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
       reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act);
@@ -540,13 +576,16 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
   const int variant = option_gemm_variant();
-#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC) \
-  launch_pipe2<WM, WN, FM, FN, XS, OCC>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
+#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...) \
+  launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
   if (variant != 2 && (k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 5);
-    if (variant >= 30 && variant <= 35) shape = variant - 30;
+    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 6);
+    if (variant >= 30 && variant <= 36) shape = variant - 30;
+    // the K-split shapes need the K tiles to divide between the groups (and the scale / bias dwords, two groups each)
+    if (shape == 6 && k_in % 256 != 0) shape = 5;
     switch (shape) {
+      case 6: return GQ_PIPE2(2, 2, 2, 1, 3, 1, 2);  // 128 x 64, 2 x 4 waves splitting K
       case 0: return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
       case 1: return GQ_PIPE2(1, 4, 8, 1, 3, 1);  // 256 x 128, 4 waves of 256 x 32
       case 2: return GQ_PIPE2(1, 4, 4, 1, 3, 2);  // 128 x 128, 4 waves of 128 x 32, two workgroups per CU

@@ -110,14 +110,15 @@ def test_gemm_edge_shapes(hip, device, oracle, n_out, k_in, gs, m_rows):
             assert normalised_error(y, y_ref) <= TOL, (entry, with_bias)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 30, 31, 32, 33, 34, 35])
+@pytest.mark.parametrize("variant", [1, 2, 30, 31, 32, 33, 34, 35, 36])
 def test_gemm_every_kernel_shape(hip, device, oracle, variant):
-    """Each tile shape of the pipelined kernel (30..35), the LDS-staged tile kernel (2) and the
+    """Each tile shape of the pipelined kernel (30..36; 36 splits K between two groups of waves and
+    falls back to 35 when the K tiles do not divide), the LDS-staged tile kernel (2) and the
     generic kernel (1) on ragged problems, including a weight with an odd number of groups per row
     (which the pipelined kernel hands to the tile kernel)."""
     try:
         hip.set_option("gemm_variant", variant)
-        for n_out, k_in, gs, m_rows in ((300, 1024, 64, 260), (130, 448, 32, 70), (96, 192, 64, 33)):
+        for n_out, k_in, gs, m_rows in ((300, 1024, 64, 260), (130, 448, 32, 70), (96, 192, 64, 33), (200, 768, 128, 100)):
             x, packed, scale, bias, ob, y_ref = _case(oracle, n_out, k_in, gs, m_rows, 41, True)
             y = _call(hip, "gq_gemm_f16", x, packed, scale, bias, ob, n_out, k_in, gs, device)
             assert np.isfinite(y).all()
