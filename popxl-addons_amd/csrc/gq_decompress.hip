@@ -148,6 +148,61 @@ __global__ __launch_bounds__(kThreads) void decompress_transposed_kernel(
   }
 }
 
+// Transposed result, fast path: a workgroup expands a tile of 128 rows x 128 columns.
+// Phase 1: thread (quarter q, row pair rp) loads the 16 bytes = 32 codes of quarter q of rows
+// 2 rp and 2 rp + 1, and computes every column for both rows at once as the two halves of
+// packed fp16 instructions (their scales and biases differ: s2 = (row a, row b)); the pair goes
+// to LDS column c as one 32-bit word.  Phase 2: a thread reads 8 consecutive rows of a column
+// (16 bytes) and stores them; 16 threads cover the 256 contiguous bytes of a column of the tile.
+// LDS: column c starts at c * 272 bytes; the row pair rp of a column of quarter q sits at word
+// rp ^ (16 q), so that the 64 lanes of a wave (4 quarters x 16 row pairs) write 64 different banks.
+constexpr int kFastTile = 128, kFastStride = 272;
+__global__ __launch_bounds__(256) void decompress_transposed_tile_kernel(
+    const uint16_t *__restrict__ packed, const half_t *__restrict__ scale, const half_t *__restrict__ bias,
+    half_t *__restrict__ out_t, int64_t rows, int64_t words_per_row, int n_ids) {
+  __shared__ __attribute__((aligned(16))) char tile[kFastTile * kFastStride];
+  const int t = threadIdx.x, q = t & 3, rp = t >> 2;
+  const int64_t row0 = (int64_t)blockIdx.y * kFastTile, word0 = (int64_t)blockIdx.x * (kFastTile / 4);
+  const int64_t n_groups = words_per_row / n_ids;
+  {
+    // rows past the end repeat the last one (their results are never stored)
+    const int64_t ra = min(row0 + 2 * rp, rows - 1), rb = min(row0 + 2 * rp + 1, rows - 1);
+    const int64_t word = word0 + q * 8, group = word / n_ids;
+    const uint4_t da = *reinterpret_cast<const uint4_t *>(packed + ra * words_per_row + word);
+    const uint4_t db = *reinterpret_cast<const uint4_t *>(packed + rb * words_per_row + word);
+    const half2_t s2 = {scale[ra * n_groups + group], scale[rb * n_groups + group]};
+    const half2_t b2 = {bias[ra * n_groups + group], bias[rb * n_groups + group]};
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    char *dst = tile + (q * 32) * kFastStride + (rp ^ (q << 4)) * 4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      // uint16 word 2k (low halves) and 2k + 1 (high halves) of both rows: (row a, row b)
+      const uint32_t both[2] = {__builtin_amdgcn_perm(db[k], da[k], 0x05040100u),
+                                __builtin_amdgcn_perm(db[k], da[k], 0x07060302u)};
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t pair = ((both[u] >> (12 - 4 * j)) & 0x000F000Fu) | 0x64006400u;
+          const half2_t code = as_half2(pair) - k1024;  // exact
+          const half2_t prod = code * s2;               // rounded to fp16
+          const half2_t v = prod + b2;                  // rounded to fp16
+          *reinterpret_cast<uint32_t *>(dst + ((2 * k + u) * 4 + j) * kFastStride) = as_u32(v);
+        }
+    }
+  }
+  __syncthreads();
+  const int rg = t & 15;  // rows 8 rg .. 8 rg + 7 of the tile
+  const int64_t row = row0 + rg * 8;
+  if (row >= rows) return;  // (rows is a multiple of 8)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int c = (t >> 4) + 16 * i;
+    const uint4_t v = *reinterpret_cast<const uint4_t *>(tile + c * kFastStride + ((4 * rg) ^ ((c >> 5) << 4)) * 4);
+    __builtin_nontemporal_store(v, reinterpret_cast<uint4_t *>(out_t + (word0 * 4 + c) * rows + row));
+  }
+}
+
 template <int THREADS, int WORDS, int UNROLL, bool NT_LOAD, bool NT_STORE>
 void launch_fast(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
                  int64_t n_words16, int shift, int64_t max_blocks, hipStream_t stream) {
@@ -168,6 +223,17 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
   if (n_words == 0) return GQ_OK;
   if (transposed) {
     const int64_t words_per_row = n_groups * n_ids;
+    // tiles of 128 x 128 with 16-byte accesses throughout
+    if (words_per_row % (kFastTile / 4) == 0 && n_ids % 8 == 0 && rows % 8 == 0 && (uintptr_t)packed % 16 == 0 &&
+        (uintptr_t)out % 16 == 0 && option_decompress_variant() != 900) {
+      const int64_t gx = words_per_row / (kFastTile / 4), gy = (rows + kFastTile - 1) / kFastTile;
+      if (gy > 65535 || gx > 0x7fffffff)
+        return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: tensor too large (rows=%lld)", (long long)rows);
+      decompress_transposed_tile_kernel<<<dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream>>>(
+          packed, reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
+          reinterpret_cast<half_t *>(out), rows, words_per_row, (int)n_ids);
+      return check_launch("decompress_transposed_tile_kernel");
+    }
     const int64_t gx = (words_per_row + kTileWords - 1) / kTileWords, gy = (rows + kTileRows - 1) / kTileRows;
     if (gy > 65535) return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: rows=%lld exceeds 65535*64", (long long)rows);
     decompress_transposed_kernel<<<dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), 0, stream>>>(

@@ -82,6 +82,33 @@ def test_ragged_shapes_all_dims(hip, device, oracle, rows, n_groups, n_ids):
     assert_bits_equal(got, want, "rank-2 scale/bias")
 
 
+@pytest.mark.parametrize("rows", [8, 136, 200, 256])
+@pytest.mark.parametrize("n_groups,n_ids", [(4, 8), (3, 32), (2, 16), (16, 16), (1, 64)])
+def test_transposed_tile_kernel(hip, device, oracle, rows, n_groups, n_ids):
+    """dim=0 through the 128 x 128 tile kernel (columns a multiple of 128, rows a multiple of 8,
+    8 or more uint16 per group): bit-exact, the forced simple kernel gives the same, and nothing
+    is written outside the result."""
+    rng = np.random.default_rng(rows * 100 + n_groups * 10 + n_ids)
+    packed = rng.integers(0, 65536, (rows, n_groups, n_ids), dtype=np.uint16)
+    scale = rng.normal(0, 0.01, (rows, n_groups, 1)).astype(np.float16)
+    bias = rng.normal(0, 0.1, (rows, n_groups, 1)).astype(np.float16)
+    want_t = oracle.c_decompress(packed, scale, bias).T
+    assert_bits_equal(_run(packed, scale, bias, device, 0), want_t, "tile kernel")
+    try:
+        hip.set_option("decompress_variant", 900)
+        assert_bits_equal(_run(packed, scale, bias, device, 0), want_t, "simple kernel")
+    finally:
+        hip.set_option("decompress_variant", 0)
+    p_dev, s_dev, b_dev = to_dev(packed, device), to_dev(scale, device), to_dev(bias, device)
+    buf = torch.full((want_t.size + 128,), 123.0, dtype=torch.float16, device=device)
+    hip.call("gq_decompress_f16_transposed", p_dev.data_ptr(), s_dev.data_ptr(), b_dev.data_ptr(), buf.data_ptr() + 128,
+             rows, n_groups, n_ids, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    res = buf.cpu().numpy()
+    assert_bits_equal(res[64 : 64 + want_t.size].reshape(want_t.shape), want_t, "guarded buffer")
+    assert np.all(res[:64] == 123.0) and np.all(res[64 + want_t.size :] == 123.0), "wrote out of bounds"
+
+
 def test_every_kernel_variant_and_alignment(hip, device, oracle):
     rng = np.random.default_rng(8)
     packed = rng.integers(0, 65536, (67, 9, 16), dtype=np.uint16)
