@@ -162,7 +162,8 @@ __global__ __launch_bounds__(256) void decompress_transposed_tile_kernel(
     half_t *__restrict__ out_t, int64_t rows, int64_t words_per_row, int n_ids) {
   __shared__ __attribute__((aligned(16))) char tile[kFastTile * kFastStride];
   const int t = threadIdx.x, q = t & 3, rp = t >> 2;
-  const int64_t row0 = (int64_t)blockIdx.y * kFastTile, word0 = (int64_t)blockIdx.x * (kFastTile / 4);
+  // (row tiles vary fastest: workgroups that run together write neighbouring stretches of the same columns)
+  const int64_t row0 = (int64_t)blockIdx.x * kFastTile, word0 = (int64_t)blockIdx.y * (kFastTile / 4);
   const int64_t n_groups = words_per_row / n_ids;
   {
     // rows past the end repeat the last one (their results are never stored)
@@ -227,9 +228,9 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
     if (words_per_row % (kFastTile / 4) == 0 && n_ids % 8 == 0 && rows % 8 == 0 && (uintptr_t)packed % 16 == 0 &&
         (uintptr_t)out % 16 == 0 && option_decompress_variant() != 900) {
       const int64_t gx = words_per_row / (kFastTile / 4), gy = (rows + kFastTile - 1) / kFastTile;
-      if (gy > 65535 || gx > 0x7fffffff)
-        return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: tensor too large (rows=%lld)", (long long)rows);
-      decompress_transposed_tile_kernel<<<dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream>>>(
+      if (gx > 65535 || gy > 0x7fffffff)
+        return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: tensor too large (columns=%lld)", (long long)words_per_row * 4);
+      decompress_transposed_tile_kernel<<<dim3((unsigned)gy, (unsigned)gx), dim3(256), 0, stream>>>(
           packed, reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
           reinterpret_cast<half_t *>(out), rows, words_per_row, (int)n_ids);
       return check_launch("decompress_transposed_tile_kernel");
