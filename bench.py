@@ -355,6 +355,20 @@ def main():
         same = np.array_equal(o.cpu().numpy().view(np.uint16), cpu_out.view(np.uint16))
         extra["gpu_equals_cpu_baseline_bits"] = bool(same)
         log(f"  {cpu['value']:.3f} GB/s on 1 core; GPU output bit-identical: {same}")
+    if args.only == "all":
+        # the same weight with the result transposed (dim=0 of the operator)
+        outs_t = [torch.empty((16384, 4096), dtype=torch.float16, device=device) for _ in dec["sets"]]
+
+        def step_t(i):
+            p, s, b, _ = dec["sets"][i % len(outs_t)]
+            hip.call("gq_decompress_f16_transposed", p.data_ptr(), s.data_ptr(), b.data_ptr(), outs_t[i % len(outs_t)].data_ptr(),
+                     4096, 256, 16, stream_handle())
+
+        ms_t = time_launches(step_t, 100, 10)
+        extra["decompress_transposed"] = {"rows": 4096, "cols": 16384, "us": ms_t * 1e3, "gbs": dec["bytes"] / ms_t / 1e6,
+                                          "hbm_frac": dec["bytes"] / ms_t / 1e6 / HBM_PEAK_GBS}
+        log(f"  transposed: {ms_t * 1e3:.1f} us, {dec['bytes'] / ms_t / 1e6:.0f} GB/s ({dec['bytes'] / ms_t / 1e6 / HBM_PEAK_GBS:.1%})")
+        del outs_t
     del dec["sets"]
     torch.cuda.empty_cache()
 
