@@ -192,6 +192,18 @@ class LinearGQ:
         )
         return fused
 
+    def prepacked(self):
+        """The weight in the streaming layout that `_gq_hip.GemvSequence.add` accepts in place of the
+        three variables (a device copy made by gq_gemv_prepack_f16; dim=0, group_size 64 and input
+        features a multiple of 512 only).  The layer keeps its variables; make the copy again after
+        `load_weights`."""
+        if self.dim != 0:
+            raise NotImplementedError("LinearGQ.prepacked: only dim=0 layers feed the GEMV sequence kernel")
+        if self.variables is None:
+            raise ValueError("LinearGQ.prepacked: the layer has no variables yet (build it or call init_variables)")
+        v = self.variables
+        return _gq_hip.prepack_gemv(v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data)
+
     # ------------------------------------------------------------------------- weight mapping
 
     @staticmethod

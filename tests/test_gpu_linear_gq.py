@@ -142,6 +142,39 @@ def test_fused_qkv_equals_separate_projections(hip, device, batch):
     assert_bits_equal(fused(x).cpu().numpy(), want.cpu().numpy())
 
 
+def test_prepacked_layer_in_a_sequence(hip, device):
+    """LinearGQ.prepacked(): the layer's weight in the streaming layout, run as entries of a GEMV
+    sequence (up-projection with GELU, then the down-projection that waits for it), gives what the
+    layers give when called one after the other."""
+    from popxl_addons._gq_hip import GemvSequence
+
+    hidden, ffn, group_size = 512, 1536, 64
+    torch.manual_seed(6)
+    layers = []
+    for n_in, n_out in ((hidden, ffn), (ffn, hidden)):
+        nn_layer = torch.nn.Linear(n_in, n_out)
+        layer = LinearGQ(n_out, bias=True, group_size=group_size, dim=0)
+        variables = layer.init_variables(n_in, torch.float16, device)
+        layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=0))
+        layers.append(layer)
+    up, down = layers
+    x = torch.randn((2, hidden), device=device, dtype=torch.float16)
+    want = down(up.build(x, activation="gelu_tanh"))
+    y_up = torch.empty((2, ffn), dtype=torch.float16, device=device)
+    y_down = torch.empty((2, hidden), dtype=torch.float16, device=device)
+    seq = GemvSequence(device)
+    first = seq.add(x, up.prepacked(), None, None, y_up, up.variables.bias.data, activation="gelu_tanh")
+    seq.add(y_up, down.prepacked(), None, None, y_down, down.variables.bias.data, wait_for=first)
+    seq.run()
+    torch.cuda.synchronize()
+    assert int(seq.status.item()) == 0
+    # the sequence kernel and the single-call kernels sum in different orders
+    err = (y_down.float() - want.float()).abs().max().item() / want.float().abs().max().item()
+    assert err <= 1e-2
+    with pytest.raises(NotImplementedError):
+        LinearGQ(64, group_size=16, dim=-1).prepacked()
+
+
 def test_fuse_rejects_mismatched_layers(hip, device):
     a = LinearGQ(64, bias=True, group_size=16, dim=0)
     a.init_variables(64, torch.float16, device)
