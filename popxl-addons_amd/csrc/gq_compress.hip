@@ -40,8 +40,8 @@ __device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float scale_f3
   return (uint32_t)c;
 }
 
-// LANES lanes share one group; each lane holds 8 consecutive elements (one 16-byte load) and
-// writes the two uint16 words made from them as one 32-bit store.  group_size = 8 * LANES.
+// LANES lanes share one group; each lane holds 8 (or 16) consecutive elements (one or two 16-byte
+// loads) and writes the uint16 words made from them as one 32-bit (64-bit) store.
 // The kernel is bound by instruction issue, not by HBM, so the work is done two elements per
 // instruction wherever a packed fp16 form exists (the roundings are those of the scalar forms).
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
@@ -59,25 +59,35 @@ __device__ __forceinline__ half2_t pk_max(half2_t a, half2_t b) {
   return r;
 }
 
-template <int LANES>
+// V: 16-byte vectors per lane (1: 8 elements, group_size = 8 LANES; 2: 16 elements, group_size =
+// 16 LANES -- half the lanes per group: one shuffle round less, and the scale, reciprocal and
+// store of the group's statistics amortised over twice the elements)
+template <int LANES, int V>
 __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__restrict__ t, uint32_t *__restrict__ packed,
                                                             half_t *__restrict__ scale, half_t *__restrict__ bias,
                                                             int32_t *__restrict__ flag, int64_t n_items) {
   const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   const bool live = item < n_items;
-  uint4_t q = {0u, 0u, 0u, 0u};
-  if (live) q = __builtin_nontemporal_load(t + item);
-  half2_t h[4];
+  half2_t h[4 * V];
   ushort2_t exponents = {0, 0};  // maximum of the exponent fields: 0x7c00 = Inf or NaN seen
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const uint32_t w = q[d];  // (a bit cast straight from a vector element reads element 0)
-    h[d] = __builtin_bit_cast(half2_t, w);
-    const uint32_t e = w & 0x7c007c00u;
-    exponents = __builtin_elementwise_max(exponents, __builtin_bit_cast(ushort2_t, e));
+  for (int v = 0; v < V; ++v) {
+    uint4_t q = {0u, 0u, 0u, 0u};
+    if (live) q = __builtin_nontemporal_load(t + item * V + v);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t w = q[d];  // (a bit cast straight from a vector element reads element 0)
+      h[4 * v + d] = __builtin_bit_cast(half2_t, w);
+      const uint32_t e = w & 0x7c007c00u;
+      exponents = __builtin_elementwise_max(exponents, __builtin_bit_cast(ushort2_t, e));
+    }
   }
-  const half2_t mx = pk_max(pk_max(h[0], h[1]), pk_max(h[2], h[3]));
-  const half2_t mn = pk_min(pk_min(h[0], h[1]), pk_min(h[2], h[3]));
+  half2_t mx = pk_max(pk_max(h[0], h[1]), pk_max(h[2], h[3]));
+  half2_t mn = pk_min(pk_min(h[0], h[1]), pk_min(h[2], h[3]));
+  if (V == 2) {
+    mx = pk_max(mx, pk_max(pk_max(h[4], h[5]), pk_max(h[6], h[7])));
+    mn = pk_min(mn, pk_min(pk_min(h[4], h[5]), pk_min(h[6], h[7])));
+  }
   // (min, max) of the group travel through the shuffles as one register; the whole wave executes
   // them, items of one group are LANES consecutive lanes
   half2_t p = {mn[0] < mn[1] ? mn[0] : mn[1], mx[0] > mx[1] ? mx[0] : mx[1]};
@@ -95,9 +105,9 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
   const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
   const float recip = __builtin_amdgcn_rcpf(sc32);
   const half2_t lo_pair = {lo, lo}, ceiling = {(half_t)1039.0f, (half_t)1039.0f}, magic = {(half_t)1024.0f, (half_t)1024.0f};
-  uint32_t m[4];  // codes of elements (2d, 2d + 1) at bits 3:0 and 19:16
+  uint32_t m[4 * V];  // codes of elements (2d, 2d + 1) at bits 3:0 and 19:16
 #pragma unroll
-  for (int d = 0; d < 4; ++d) {
+  for (int d = 0; d < 4 * V; ++d) {
     const half2_t diff = h[d] - lo_pair;
     const half2_t quot = {divide(diff[0], sc32, recip), divide(diff[1], sc32, recip)};
     // quot + 1024 rounds to an integer, ties to even (the ulp of fp16 at 1024 is 1): that is
@@ -106,10 +116,19 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
     const half2_t biased = pk_min(quot + magic, ceiling);
     m[d] = __builtin_bit_cast(uint32_t, biased) & 0x000F000Fu;
   }
-  const uint32_t w0 = ((m[0] << 12) | (m[0] >> 8) | (m[1] << 4) | (m[1] >> 16)) & 0xFFFFu;
-  const uint32_t w1 = ((m[2] << 12) | (m[2] >> 8) | (m[3] << 4) | (m[3] >> 16)) & 0xFFFFu;
+  uint32_t word[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t w0 = ((m[4 * v] << 12) | (m[4 * v] >> 8) | (m[4 * v + 1] << 4) | (m[4 * v + 1] >> 16)) & 0xFFFFu;
+    const uint32_t w1 = ((m[4 * v + 2] << 12) | (m[4 * v + 2] >> 8) | (m[4 * v + 3] << 4) | (m[4 * v + 3] >> 16)) & 0xFFFFu;
+    word[v] = w0 | (w1 << 16);
+  }
   if (live) {
-    packed[item] = w0 | (w1 << 16);
+    if (V == 1) {
+      packed[item] = word[0];
+    } else {
+      *reinterpret_cast<uint2_t *>(packed + item * 2) = uint2_t{word[0], word[V - 1]};
+    }
     if ((item & (LANES - 1)) == 0) {
       scale[item / LANES] = sc;
       bias[item / LANES] = lo;
@@ -154,7 +173,9 @@ __global__ __launch_bounds__(kThreads) void compress_generic_kernel(const half_t
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
                     int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream) {
   const int64_t groups_total = rows * n_groups;
-  const int lanes = (int)(group_size / 8);
+  // 16 elements per lane where the group allows it, else 8
+  const int per_lane = group_size % 16 == 0 && ((uintptr_t)packed % 8) == 0 ? 16 : 8;
+  const int lanes = (int)(group_size / per_lane);
   const bool fast = group_size % 8 == 0 && (lanes & (lanes - 1)) == 0 && lanes <= 64 && ((uintptr_t)t % 16) == 0 &&
                     ((uintptr_t)packed % 4) == 0;
   if (fast) {
@@ -165,15 +186,21 @@ int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16
     const uint4_t *src = reinterpret_cast<const uint4_t *>(t);
     uint32_t *dst = reinterpret_cast<uint32_t *>(packed);
     half_t *s = reinterpret_cast<half_t *>(scale), *b = reinterpret_cast<half_t *>(bias);
+#define GQ_COMPRESS(L)                                                                                  \
+  do {                                                                                                  \
+    if (per_lane == 16) compress_kernel<L, 2><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); \
+    else compress_kernel<L, 1><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items);              \
+  } while (0)
     switch (lanes) {
-      case 1: compress_kernel<1><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      case 2: compress_kernel<2><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      case 4: compress_kernel<4><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      case 8: compress_kernel<8><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      case 16: compress_kernel<16><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      case 32: compress_kernel<32><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
-      default: compress_kernel<64><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 1: GQ_COMPRESS(1); break;
+      case 2: GQ_COMPRESS(2); break;
+      case 4: GQ_COMPRESS(4); break;
+      case 8: GQ_COMPRESS(8); break;
+      case 16: GQ_COMPRESS(16); break;
+      case 32: GQ_COMPRESS(32); break;
+      default: GQ_COMPRESS(64); break;
     }
+#undef GQ_COMPRESS
     return check_launch("compress_kernel");
   }
   const int64_t blocks = (groups_total + kThreads - 1) / kThreads;

@@ -84,6 +84,29 @@ def test_device_compress_bit_exact(hip, device, oracle, group_size):
     assert_bits_equal(b.cpu().numpy(), bw, "bias")
 
 
+def test_device_compress_output_alignment(hip, device, oracle):
+    """A packed output that is only 4-byte aligned takes the kernel with 8 elements per lane
+    (32-bit stores) instead of 16 (64-bit stores): same bits."""
+    rng = np.random.default_rng(77)
+    w = rng.normal(0, 0.02, (40, 512)).astype(np.float16)
+    pw, sw, bw = oracle.c_compress(w, 64)
+    wd = to_dev(w, device)
+    buf = torch.zeros(pw.size + 8, dtype=torch.uint16, device=device)
+    scale = torch.empty(sw.shape, dtype=torch.float16, device=device)
+    bias = torch.empty(bw.shape, dtype=torch.float16, device=device)
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    for offset in (0, 2):  # in uint16 elements: 0 and 4 bytes
+        buf.zero_()
+        hip.call("gq_compress_f16", wd.data_ptr(), buf.data_ptr() + 2 * offset, scale.data_ptr(), bias.data_ptr(),
+                 flag.data_ptr(), 40, 8, 64, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = buf.cpu().numpy()
+        assert np.array_equal(got[offset : offset + pw.size].reshape(pw.shape), pw), offset
+        assert not got[:offset].any() and not got[offset + pw.size :].any()
+        assert_bits_equal(scale.cpu().numpy(), sw, "scale")
+        assert_bits_equal(bias.cpu().numpy(), bw, "bias")
+
+
 def test_device_compress_config2_and_nonfinite(hip, device, oracle):
     w = config2_weight(1024, 16384, seed=4)
     p, s, b = group_quantize_compress(to_dev(w, device), 64)
