@@ -85,7 +85,7 @@ def test_compress_equals_oracle(oracle, dtype, group_size, dim):
 
 
 def test_config1_round_trip(oracle):
-    """BASELINE config 1: 1024 x 1024 ~ N(0, 0.02), group 64; |error| <= scale/2 (+ fp16 slack)."""
+    """Benchmark configuration 1: 1024 x 1024 ~ N(0, 0.02), group 64; |error| <= scale/2 (+ fp16 slack)."""
     rng = np.random.default_rng(1)
     w = rng.normal(0, 0.02, (1024, 1024)).astype(np.float16)
     packed, scale, bias = group_quantize_compress_numpy(w, 64)
