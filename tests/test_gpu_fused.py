@@ -272,6 +272,48 @@ def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
     assert "streaming layout" in str(e.value)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_gemv_sequence_random_graphs(hip, device, oracle, seed):
+    """Seeded random sequences: shapes with ragged row counts and 1 - 16 chunks, batch 1 - 4, each
+    entry reading the activations or the output of a random earlier entry (and waiting for it),
+    random epilogues, both weight layouts mixed.  Every entry is checked against the oracle applied
+    to the input the device actually had."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    rng = np.random.default_rng(1000 + seed)
+    m_rows = int(rng.integers(1, 5))
+    widths = [512 * int(rng.integers(1, 5)) for _ in range(3)] + [512 * int(rng.integers(5, 17))]
+    n_entries = int(rng.integers(6, 15))
+    x0 = activations(m_rows, widths[0], seed)
+    seq = GemvSequence(device)
+    feeds = [(to_dev(x0, device), widths[0], None)]  # (device tensor, width, producing entry)
+    entries = []
+    for i in range(n_entries):
+        x_dev, k_in, producer = feeds[int(rng.integers(0, len(feeds)))]
+        n_out = int(rng.choice(widths)) if rng.random() < 0.6 else int(rng.integers(1, 1500))
+        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        ob = rng.normal(0, 0.1, (n_out,)).astype(np.float16) if rng.random() < 0.5 else None
+        act = [None, "relu", "gelu_tanh"][int(rng.integers(0, 3))]
+        pd, sd, bd = (to_dev(a, device) for a in (packed, scale, bias))
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        args = (prepack_gemv(pd, sd, bd), None, None) if rng.random() < 0.5 else (pd, sd, bd)
+        seq.add(x_dev, *args, y, None if ob is None else to_dev(ob, device), wait_for=producer, activation=act)
+        entries.append((x_dev, y, oracle.np_decompress(packed, scale, bias), ob, act))
+        if n_out % 512 == 0:
+            feeds.append((y, n_out, i))
+    for _ in range(2):
+        for _x, y, *_rest in entries:
+            y.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        for i, (x_dev, y, w_dec, ob, act) in enumerate(entries):
+            got = y.cpu().numpy()
+            assert np.isfinite(got).all(), (seed, i)
+            assert normalised_error(got, oracle.np_linear(x_dev.cpu().numpy(), w_dec, ob, act)) <= TOL, (seed, i)
+
+
 def test_gemv_sequence_fallback_and_graph(hip, device, oracle):
     """Shapes outside the persistent kernel (group 32) run entry by entry; the persistent kernel
     replays correctly from a captured graph."""
