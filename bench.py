@@ -306,9 +306,6 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB device copy (known traffic) for scaling profiler byte counters")
-    ap.add_argument("--decompress-variant", type=int, default=0)
-    ap.add_argument("--gemv-variant", type=int, default=0)
-    ap.add_argument("--gemm-variant", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -322,9 +319,6 @@ def main():
         sys.exit("bench.py: no HIP device visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    hip.set_option("decompress_variant", args.decompress_variant)
-    hip.set_option("gemv_variant", args.gemv_variant)
-    hip.set_option("gemm_variant", args.gemm_variant)
     log(f"device: {torch.cuda.get_device_name(0)}")
 
     extra = {}

@@ -17,8 +17,9 @@
  *     (nothing was launched); a positive value is a `hipError_t` from the runtime.
  *     `gq_last_error()` returns a thread-local, human-readable description of the last
  *     non-zero return on the calling thread.
- *   - Functions are re-entrant, allocate nothing and keep no per-call state (one exception:
- *     gq_gemv_sequence_f16, see there); every entry point can be captured in a HIP graph.
+ *   - Functions are re-entrant, allocate nothing and keep no state between calls (one exception:
+ *     gq_gemv_sequence_f16 uses a block of progress words that the library keeps per device, see
+ *     there); there are no process-wide options.  Every entry point can be captured in a HIP graph.
  *
  * Packed layout (group_quantize_decompress.py:127-135, group_quantize_decompress_codelet.cpp:11-14)
  *   packed[r][g][i] is a little-endian uint16 holding four 4-bit codes, most significant
@@ -34,7 +35,7 @@
 extern "C" {
 #endif
 
-#define GQ_ABI_VERSION 1
+#define GQ_ABI_VERSION 2
 
 #define GQ_OK 0
 #define GQ_ERR_NULL_POINTER (-1) /* a required pointer is NULL */
@@ -54,12 +55,6 @@ int gq_abi_version(void);
 
 /* Thread-local description of the last failing call on this thread ("" if none). */
 const char *gq_last_error(void);
-
-/* Tuning/diagnostic switches, by name.  Unknown names return GQ_ERR_UNSUPPORTED.
- *   "decompress_variant"  kernel flavour of gq_decompress_f16 (0 = default)
- *   "gemv_variant"        kernel flavour of gq_gemv_f16       (0 = default)
- *   "gemm_variant"        kernel flavour of gq_gemm_f16       (0 = default) */
-int gq_set_option(const char *name, int64_t value);
 
 /*
  * Standalone decompress.  Replaces the device op created by
@@ -130,10 +125,39 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
                       int64_t k_in, int64_t group_size, int32_t activation, void *stream);
 
 /*
+ * Fused decompress + matmul, groups along the OUTPUT features: the computation of LinearGQ.build
+ * with dim = -1 or 1, the constructor default (popxl_addons/layers/linear_gq.py:26, 59-62, 99-109):
+ *   w = decompress(packed, scale, bias)      [k_in, n_out]
+ *   y[m][n] = act( sum_k x[m][k] * w[k][n] (+ out_bias[n]) )
+ * without writing w to memory.
+ *
+ *   x        [m_rows, k_in] binary16             y [m_rows, n_out] binary16
+ *   packed   [k_in, n_out / group_size, group_size / 4] uint16
+ *   scale, bias [k_in, n_out / group_size] binary16
+ *   out_bias [n_out] binary16 or NULL;  activation: GQ_ACT_*
+ * Same accumulation and tolerance as gq_linear_act_f16.  Requirements: group_size % 4 == 0,
+ * n_out % group_size == 0; the fast kernels need a power-of-two group_size >= 32, n_out % 32 == 0
+ * and a 16-byte aligned packed (plus k_in % 64 == 0 and a 16-byte aligned x for m_rows > 16); other
+ * shapes run a slower generic kernel with the same results.
+ *
+ * For m_rows <= 16 the contraction is split between workgroups, whose binary32 partial sums meet
+ * in `workspace`: device memory, 16-byte aligned, at least gq_linear_kn_workspace_bytes() bytes
+ * for the same sizes (0: none needed, workspace may be NULL).  Its first 16 KiB hold arrival
+ * counters: the caller zeroes them once, every call leaves them zero, so one workspace serves
+ * calls of any shape -- one at a time: calls that share a workspace must not overlap.
+ */
+int64_t gq_linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
+int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                         int64_t k_in, int64_t group_size, int32_t activation, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
+/*
  * A sequence of decode GEMVs (a layer stack) as one call.  No counterpart in the reference, where
  * a model is a chain of LinearGQ.build calls (popxl_addons/layers/linear_gq.py:99-109) compiled
  * into one static device program; this entry point is the analogue for a chain of gq_gemv_f16
- * calls: entry i computes exactly what gq_gemv_f16 would.  Dependencies between entries are
+ * calls: entry i computes what gq_gemv_f16 would, to the tolerance of the fused paths (the
+ * summation order differs).  Dependencies between entries are
  * declared, not implied: entry i starts only after the first wait_entries[i] entries of the
  * sequence have completed (0 <= wait_entries <= i; 0 = no dependency, i = every earlier entry).
  * Set it past the entry that produces x or out_bias of entry i.  Entries may otherwise overlap
@@ -148,8 +172,22 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
  *   descs_device  device copy of the same `count` entries (read by the kernel)
  *   status        device int32 or NULL; set to 1 if the kernel gave up waiting for earlier entries
  *                 (it then still terminates; results are invalid).  The caller zeroes it.
- * The persistent kernel keeps its progress counters in device globals: at most one sequence may
- * run on a device at a time.
+ *
+ * The persistent kernel launches one workgroup per compute unit and relies on all of them being
+ * resident together: nothing else should occupy the compute units while it runs.  Every wait is
+ * bounded: a poller that sees no progress `spin_limit` polls in a row gives up, sets *status and
+ * lets the kernel drain (results are then invalid, the progress words are back at zero).
+ *
+ * gq_gemv_sequence_f16     keeps the per-workgroup progress words in a block that the library
+ *                          holds per device: at most ONE sequence may run on a device at a time.
+ * gq_gemv_sequence_ws_f16  takes them from `workspace` (device memory, 256-byte aligned,
+ *                          gq_gemv_sequence_workspace_bytes() bytes, zeroed by the caller once; the
+ *                          kernel leaves it zeroed), so that the library holds no state for the
+ *                          call: sequences with workspaces of their own may be enqueued on
+ *                          different streams and captured in different graphs, as long as the
+ *                          caller orders them (events) so that two persistent kernels never run at
+ *                          the same time -- each needs every compute unit.  spin_limit <= 0 selects
+ *                          the default (2^18 polls).
  */
 typedef struct gq_gemv_desc {
   const uint16_t *x;        /* [m_rows, k_in] binary16 */
@@ -186,6 +224,10 @@ int gq_gemv_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uin
 
 int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
                          int32_t *status, void *stream);
+int64_t gq_gemv_sequence_workspace_bytes(void);
+int gq_gemv_sequence_ws_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                            int32_t *status, void *workspace, int64_t workspace_bytes, int64_t spin_limit,
+                            void *stream);
 
 /*
  * Device-side compress for binary16 input: bit-identical packed/scale/bias to
@@ -199,6 +241,16 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
  * (the reference raises ValueError there, :182-183); outputs are then unspecified.
  */
 int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,
+                    int32_t *nonfinite_flag, int64_t rows, int64_t n_groups, int64_t group_size,
+                    void *stream);
+
+/*
+ * The same for binary32 input, which is what LinearGQ.torch_mapping feeds the packer
+ * (popxl_addons/layers/linear_gq.py:130: nn_layer.weight.T, float32): max / min are taken in
+ * binary32 and cast to binary16, the scale is binary16 arithmetic, (x - bias) / scale is a binary32
+ * subtraction and division (group_quantize_decompress.py:186-192).
+ */
+int gq_compress_f32(const float *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,
                     int32_t *nonfinite_flag, int64_t rows, int64_t n_groups, int64_t group_size,
                     void *stream);
 

@@ -1,7 +1,6 @@
 // C-ABI layer of libgq_hip: argument validation, error text, dispatch to the launchers.
 // Shape rules follow GroupQuantizeDecompressOp::setup (group_quantize_decompress.cpp:35-77)
 // and LinearGQ.build (popxl_addons/layers/linear_gq.py:58-110).
-#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -12,7 +11,6 @@ namespace gq {
 
 namespace {
 thread_local char g_error[512] = "";
-std::atomic<int> g_decompress_variant{0}, g_gemv_variant{0}, g_gemm_variant{0};
 }  // namespace
 
 int fail(int code, const char *fmt, ...) {
@@ -28,10 +26,6 @@ int check_launch(const char *what) {
   if (e == hipSuccess) return GQ_OK;
   return fail((int)e, "%s: %s", what, hipGetErrorString(e));
 }
-
-int option_decompress_variant() { return g_decompress_variant.load(std::memory_order_relaxed); }
-int option_gemv_variant() { return g_gemv_variant.load(std::memory_order_relaxed); }
-int option_gemm_variant() { return g_gemm_variant.load(std::memory_order_relaxed); }
 
 namespace {
 
@@ -84,15 +78,6 @@ extern "C" {
 int gq_abi_version(void) { return GQ_ABI_VERSION; }
 
 const char *gq_last_error(void) { return gq::g_error; }
-
-int gq_set_option(const char *name, int64_t value) {
-  if (!name) return gq::fail(GQ_ERR_NULL_POINTER, "gq_set_option: name is NULL");
-  if (!strcmp(name, "decompress_variant")) gq::g_decompress_variant = (int)value;
-  else if (!strcmp(name, "gemv_variant")) gq::g_gemv_variant = (int)value;
-  else if (!strcmp(name, "gemm_variant")) gq::g_gemm_variant = (int)value;
-  else return gq::fail(GQ_ERR_UNSUPPORTED, "gq_set_option: unknown option '%s'", name);
-  return GQ_OK;
-}
 
 int gq_decompress_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
                       int64_t rows, int64_t n_groups, int64_t n_ids, void *stream) {
@@ -154,8 +139,61 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
                          (hipStream_t)stream);
 }
 
-int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
-                         int32_t *status, void *stream) {
+int64_t gq_linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (m_rows < 0 || n_out < 0 || k_in < 0 || group_size <= 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_kn_workspace_bytes: negative size");
+  return gq::linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
+}
+
+// argument checks shared by the entry points of the [k_in, n_out] layout; 1 = proceed
+static int check_linear_kn_args(const char *who, const uint16_t *x, int64_t m_rows, const uint16_t *packed,
+                                const uint16_t *scale, const uint16_t *bias, const uint16_t *out_bias, uint16_t *y,
+                                int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation) {
+  if (m_rows < 0 || n_out < 0 || k_in < 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "%s: negative size (m_rows=%lld n_out=%lld k_in=%lld)", who, (long long)m_rows,
+                    (long long)n_out, (long long)k_in);
+  if (group_size <= 0 || group_size % 4 != 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "%s: group_size=%lld must be a positive multiple of 4", who, (long long)group_size);
+  if (n_out % group_size != 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "%s: n_out=%lld is not a multiple of group_size=%lld", who, (long long)n_out,
+                    (long long)group_size);
+  if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "%s: unknown activation %d", who, (int)activation);
+  if (m_rows == 0 || n_out == 0) return GQ_OK;
+  if (!y) return gq::fail(GQ_ERR_NULL_POINTER, "%s: y is NULL", who);
+  if (k_in > 0 && (!x || !packed || !scale || !bias))
+    return gq::fail(GQ_ERR_NULL_POINTER, "%s: x/packed/scale/bias must not be NULL", who);
+  if (gq::misaligned(x, 2) || gq::misaligned(packed, 2) || gq::misaligned(scale, 2) || gq::misaligned(bias, 2) ||
+      gq::misaligned(out_bias, 2) || gq::misaligned(y, 2))
+    return gq::fail(GQ_ERR_MISALIGNED, "%s: pointers must be 2-byte aligned", who);
+  if (m_rows > (int64_t)1 << 30 || n_out > (int64_t)1 << 30 || k_in > (int64_t)1 << 30)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "%s: a dimension exceeds 2^30", who);
+  return 1;
+}
+
+int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                         int64_t group_size, int32_t activation, void *workspace, int64_t workspace_bytes,
+                         void *stream) {
+  const int rc = check_linear_kn_args("gq_linear_kn_act_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in,
+                                      group_size, activation);
+  if (rc <= 0) return rc;
+  const int64_t need = gq::linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
+  if (need > 0) {
+    if (!workspace) return gq::fail(GQ_ERR_NULL_POINTER, "gq_linear_kn_act_f16: this problem needs a workspace of %lld bytes",
+                                    (long long)need);
+    if (gq::misaligned(workspace, 16))
+      return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_kn_act_f16: workspace must be 16-byte aligned");
+    if (workspace_bytes < need)
+      return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_kn_act_f16: workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+                      (long long)need);
+  }
+  return gq::launch_linear_kn(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
+                              workspace, (hipStream_t)stream);
+}
+
+static int gemv_sequence_common(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                                int32_t *status, void *workspace, int64_t spin_limit, void *stream) {
   if (count < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: negative count");
   if (count == 0) return GQ_OK;
   if (!descs || !descs_device) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_sequence_f16: descs is NULL");
@@ -191,7 +229,28 @@ int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_de
       return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: entry %lld has wait_entries=%d outside [0, %lld]",
                       (long long)i, d.wait_entries, (long long)i);
   }
-  return gq::launch_gemv_sequence(descs, descs_device, count, status, (hipStream_t)stream);
+  return gq::launch_gemv_sequence(descs, descs_device, count, status, workspace, spin_limit, (hipStream_t)stream);
+}
+
+int gq_gemv_sequence_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                         int32_t *status, void *stream) {
+  return gemv_sequence_common(descs, descs_device, count, status, nullptr, 0, stream);
+}
+
+int64_t gq_gemv_sequence_workspace_bytes(void) { return gq::gemv_sequence_workspace_bytes(); }
+
+int gq_gemv_sequence_ws_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
+                            int32_t *status, void *workspace, int64_t workspace_bytes, int64_t spin_limit,
+                            void *stream) {
+  if (count > 0) {
+    if (!workspace) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_sequence_ws_f16: workspace is NULL");
+    if (gq::misaligned(workspace, 256))
+      return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_ws_f16: workspace must be 256-byte aligned");
+    if (workspace_bytes < gq::gemv_sequence_workspace_bytes())
+      return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_ws_f16: workspace of %lld bytes, need %lld",
+                      (long long)workspace_bytes, (long long)gq::gemv_sequence_workspace_bytes());
+  }
+  return gemv_sequence_common(descs, descs_device, count, status, workspace, spin_limit, stream);
 }
 
 int64_t gq_gemv_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size) {
@@ -233,6 +292,23 @@ int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_compress_f16: more than 2^40 elements");
   return gq::launch_compress(t, packed, scale, bias, nonfinite_flag, rows, n_groups, group_size,
                              (hipStream_t)stream);
+}
+
+int gq_compress_f32(const float *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *nonfinite_flag,
+                    int64_t rows, int64_t n_groups, int64_t group_size, void *stream) {
+  if (rows < 0 || n_groups < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_compress_f32: negative size");
+  if (group_size <= 0 || group_size % 4 != 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_compress_f32: group_size=%lld must be a positive multiple of 4",
+                    (long long)group_size);
+  if (rows == 0 || n_groups == 0) return GQ_OK;
+  if (!t || !packed || !scale || !bias) return gq::fail(GQ_ERR_NULL_POINTER, "gq_compress_f32: NULL pointer argument");
+  if (gq::misaligned(t, 4) || gq::misaligned(packed, 2) || gq::misaligned(scale, 2) || gq::misaligned(bias, 2) ||
+      gq::misaligned(nonfinite_flag, 4))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_compress_f32: misaligned pointer");
+  if (rows > ((int64_t)1 << 40) / n_groups / group_size)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_compress_f32: more than 2^40 elements");
+  return gq::launch_compress_f32(t, packed, scale, bias, nonfinite_flag, rows, n_groups, group_size,
+                                 (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -12,10 +12,6 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // Maps the runtime's last launch error (if any) to a return code, recording its text.
 int check_launch(const char *what);
 
-int option_decompress_variant();
-int option_gemv_variant();
-int option_gemm_variant();
-
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -50,12 +46,21 @@ int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *
 int launch_gemv_streamed(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                          const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                          int64_t group_size, int act, hipStream_t stream);
+// workspace: the sequence's progress words (gemv_sequence_workspace_bytes() zeroed bytes), or
+// nullptr for the block the library keeps per device; spin_limit <= 0: the default
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
-                         hipStream_t stream);
+                         void *workspace, int64_t spin_limit, hipStream_t stream);
+int64_t gemv_sequence_workspace_bytes();
+int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
+int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                     const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                     int64_t group_size, int act, void *workspace, hipStream_t stream);
 int64_t gemv_prepacked_bytes(int64_t n_out, int64_t k_in);
 int launch_gemv_prepack(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
                         int64_t k_in, hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
                     int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
+int launch_compress_f32(const float *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
+                        int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
 
 }  // namespace gq

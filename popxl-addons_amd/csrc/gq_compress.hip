@@ -1,4 +1,4 @@
-// Device-side 4-bit group-quantization compress (fp16 input) for gfx950.
+// Device-side 4-bit group-quantization compress (fp16 or fp32 input) for gfx950.
 //
 // Produces the same packed / scale / bias bits as group_quantize_compress_numpy on a float16
 // array (popxl_addons/ops/group_quantize_decompress/group_quantize_decompress.py:178-196):
@@ -168,6 +168,101 @@ __global__ __launch_bounds__(kThreads) void compress_generic_kernel(const half_t
   if (bad && flag) *flag = 1;
 }
 
+// ---------------------------------------------------------------------------------------
+// fp32 input (what LinearGQ.torch_mapping feeds the packer: nn.Linear weights, linear_gq.py:130).
+// The reference promotes to fp32 there (group_quantize_decompress.py:186-192): max / min are taken
+// in fp32 and cast to fp16, the scale is fp16 arithmetic, and (x - lo) / scale is an fp32
+// subtraction and a correctly rounded fp32 division.  HBM-bound: 4 B read per element.
+// LANES lanes share a group, 8 elements (two 16-byte loads) per lane; LANES == 0: one lane per
+// group, any group_size % 4 == 0.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t quantize_f32(float v, float lo, float sc) {
+  const float quot = (v - lo) / sc;  // both rounded to fp32 (contraction is off; the division is IEEE)
+  int c = (int)__builtin_rintf(quot);
+  c = c < 0 ? 0 : (c > 15 ? 15 : c);  // no effect wherever the reference is well defined
+  return (uint32_t)c;
+}
+
+template <int LANES>
+__global__ __launch_bounds__(kThreads) void compress_f32_kernel(const float4_t *__restrict__ t, uint32_t *__restrict__ packed,
+                                                                half_t *__restrict__ scale, half_t *__restrict__ bias,
+                                                                int32_t *__restrict__ flag, int64_t n_items) {
+  const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const bool live = item < n_items;
+  float v[8];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    float4_t f = {0.f, 0.f, 0.f, 0.f};
+    if (live) f = __builtin_nontemporal_load(t + item * 2 + q);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[4 * q + e] = f[e];
+  }
+  float mx = v[0], mn = v[0];
+  bool bad = false;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bad |= (__builtin_bit_cast(uint32_t, v[e]) & 0x7f800000u) == 0x7f800000u;
+    mx = v[e] > mx ? v[e] : mx;
+    mn = v[e] < mn ? v[e] : mn;
+  }
+#pragma unroll
+  for (int off = LANES / 2; off > 0; off >>= 1) {
+    const float omx = __shfl_xor(mx, off, 64), omn = __shfl_xor(mn, off, 64);
+    mx = omx > mx ? omx : mx;
+    mn = omn < mn ? omn : mn;
+  }
+  const half_t hi = (half_t)mx, lo = (half_t)mn;
+  const half_t range = hi - lo;
+  const half_t sc = (half_t)((float)range / 15.0f);
+  const float lo32 = (float)lo;
+  // scale 0 (constant group): every code is 0; an infinite divisor gives that without a branch
+  const float sc32 = (float)sc == 0.f ? __builtin_inff() : (float)sc;
+  uint32_t w[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+    w[q] = (quantize_f32(v[4 * q], lo32, sc32) << 12) | (quantize_f32(v[4 * q + 1], lo32, sc32) << 8) |
+           (quantize_f32(v[4 * q + 2], lo32, sc32) << 4) | quantize_f32(v[4 * q + 3], lo32, sc32);
+  if (live) {
+    packed[item] = w[0] | (w[1] << 16);
+    if ((item & (LANES - 1)) == 0) {
+      scale[item / LANES] = sc;
+      bias[item / LANES] = lo;
+    }
+    if (flag && bad) *flag = 1;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void compress_f32_generic_kernel(const float *__restrict__ t,
+                                                                        uint16_t *__restrict__ packed,
+                                                                        half_t *__restrict__ scale,
+                                                                        half_t *__restrict__ bias, int32_t *__restrict__ flag,
+                                                                        int64_t n_groups_total, int group_size) {
+  const int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (g >= n_groups_total) return;
+  const float *src = t + g * group_size;
+  float mx = src[0], mn = src[0];
+  bool bad = false;
+  for (int e = 0; e < group_size; ++e) {
+    const float v = src[e];
+    bad |= (__builtin_bit_cast(uint32_t, v) & 0x7f800000u) == 0x7f800000u;
+    mx = v > mx ? v : mx;
+    mn = v < mn ? v : mn;
+  }
+  const half_t hi = (half_t)mx, lo = (half_t)mn;
+  const half_t range = hi - lo;
+  const half_t sc = (half_t)((float)range / 15.0f);
+  scale[g] = sc;
+  bias[g] = lo;
+  const float lo32 = (float)lo;
+  const float sc32 = (float)sc == 0.f ? __builtin_inff() : (float)sc;
+  for (int i = 0; i < group_size / 4; ++i) {
+    uint32_t w = 0;
+    for (int j = 0; j < 4; ++j) w = (w << 4) | quantize_f32(src[4 * i + j], lo32, sc32);
+    packed[g * (group_size / 4) + i] = (uint16_t)w;
+  }
+  if (bad && flag) *flag = 1;
+}
+
 }  // namespace
 
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
@@ -209,6 +304,38 @@ int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16
       reinterpret_cast<const half_t *>(t), packed, reinterpret_cast<half_t *>(scale),
       reinterpret_cast<half_t *>(bias), flag, groups_total, (int)group_size);
   return check_launch("compress_generic_kernel");
+}
+
+int launch_compress_f32(const float *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag, int64_t rows,
+                        int64_t n_groups, int64_t group_size, hipStream_t stream) {
+  const int64_t groups_total = rows * n_groups;
+  const int lanes = (int)(group_size / 8);
+  const bool fast = group_size % 8 == 0 && (lanes & (lanes - 1)) == 0 && lanes <= 64 && ((uintptr_t)t % 16) == 0 &&
+                    ((uintptr_t)packed % 4) == 0;
+  half_t *s = reinterpret_cast<half_t *>(scale), *b = reinterpret_cast<half_t *>(bias);
+  if (fast) {
+    const int64_t n_items = groups_total * lanes;
+    const int64_t blocks = (n_items + kThreads - 1) / kThreads;
+    if (blocks >= (int64_t)1 << 31) return fail(GQ_ERR_UNSUPPORTED, "gq_compress_f32: tensor too large");
+    const dim3 grid((unsigned)blocks), block(kThreads);
+    const float4_t *src = reinterpret_cast<const float4_t *>(t);
+    uint32_t *dst = reinterpret_cast<uint32_t *>(packed);
+    switch (lanes) {
+      case 1: compress_f32_kernel<1><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 2: compress_f32_kernel<2><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 4: compress_f32_kernel<4><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 8: compress_f32_kernel<8><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 16: compress_f32_kernel<16><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      case 32: compress_f32_kernel<32><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+      default: compress_f32_kernel<64><<<grid, block, 0, stream>>>(src, dst, s, b, flag, n_items); break;
+    }
+    return check_launch("compress_f32_kernel");
+  }
+  const int64_t blocks = (groups_total + kThreads - 1) / kThreads;
+  if (blocks >= (int64_t)1 << 31) return fail(GQ_ERR_UNSUPPORTED, "gq_compress_f32: tensor too large");
+  compress_f32_generic_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(t, packed, s, b, flag, groups_total,
+                                                                                     (int)group_size);
+  return check_launch("compress_f32_generic_kernel");
 }
 
 }  // namespace gq

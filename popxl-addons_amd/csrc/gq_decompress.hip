@@ -42,59 +42,24 @@ __device__ __forceinline__ uint4_t expand_word(uint32_t w, half2_t s2, half2_t b
   return o;
 }
 
-template <bool NT>
-__device__ __forceinline__ void store16(uint4_t *p, uint4_t v) {
-  if (NT)
-    __builtin_nontemporal_store(v, p);
-  else
-    *p = v;
-}
-
-template <typename T, bool NT>
-__device__ __forceinline__ T load_packed(const T *p) {
-  if (NT) return __builtin_nontemporal_load(p);
-  return *p;
-}
-
-// Fast path.  One work item = WORDS consecutive 32-bit words of the flattened packed tensor
-// (WORDS in {1, 2, 4}: a 4/8/16-byte load) -> WORDS 16-byte stores.  All words of an item
-// lie in one group (the launcher guarantees WORDS divides the words per group), so an item
-// needs one (scale, bias) pair.  Items are dealt to lanes so that consecutive lanes take
-// consecutive items: with WORDS == 1 every load and store instruction of a wave covers one
-// contiguous span (256 B read, 1 KiB written).  A workgroup walks the tensor with a grid
-// stride of THREADS * UNROLL items; the launcher picks the grid (one pass or persistent).
-template <int THREADS, int WORDS, int UNROLL, bool NT_LOAD, bool NT_STORE>
-__global__ __launch_bounds__(THREADS) void decompress_kernel(const uint32_t *__restrict__ packed,
-                                                             const half_t *__restrict__ scale,
-                                                             const half_t *__restrict__ bias,
-                                                             uint4_t *__restrict__ out, int64_t n_items,
-                                                             int items_per_group_shift) {
-  typedef uint32_t vec_t __attribute__((ext_vector_type(WORDS)));
-  const int64_t stride = (int64_t)gridDim.x * (THREADS * UNROLL);
-  for (int64_t base = (int64_t)blockIdx.x * (THREADS * UNROLL) + threadIdx.x; base < n_items; base += stride) {
-    vec_t w[UNROLL];
-    half_t s[UNROLL], b[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t item = base + (int64_t)u * THREADS;
-      if (item < n_items) {
-        w[u] = load_packed<vec_t, NT_LOAD>(reinterpret_cast<const vec_t *>(packed) + item);
-        const int64_t group = item >> items_per_group_shift;
-        s[u] = scale[group];
-        b[u] = bias[group];
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t item = base + (int64_t)u * THREADS;
-      if (item < n_items) {
-        const half2_t s2 = {s[u], s[u]}, b2 = {b[u], b[u]};
-        uint4_t *dst = out + item * WORDS;
-#pragma unroll
-        for (int k = 0; k < WORDS; ++k) store16<NT_STORE>(dst + k, expand_word(w[u][k], s2, b2));
-      }
-    }
-  }
+// Fast path.  One lane = one 32-bit word of the flattened packed tensor (8 codes) -> one 16-byte
+// store: every load instruction of a wave covers 256 contiguous bytes and every store 1 KiB.
+// Loads are ordinary cached loads (8 lanes share a scale/bias pair), stores are non-temporal.
+// One pass over the tensor, 512 threads per workgroup (measured against 64..1024 threads, wider
+// items per lane, non-temporal loads and persistent grids: all slower).
+constexpr int kFastThreads = 512;
+__global__ __launch_bounds__(kFastThreads) void decompress_kernel(const uint32_t *__restrict__ packed,
+                                                                  const half_t *__restrict__ scale,
+                                                                  const half_t *__restrict__ bias,
+                                                                  uint4_t *__restrict__ out, int64_t n_items,
+                                                                  int items_per_group_shift) {
+  const int64_t item = (int64_t)blockIdx.x * kFastThreads + threadIdx.x;
+  if (item >= n_items) return;
+  const uint32_t w = packed[item];
+  const int64_t group = item >> items_per_group_shift;
+  const half_t s = scale[group], b = bias[group];
+  const half2_t s2 = {s, s}, b2 = {b, b};
+  __builtin_nontemporal_store(expand_word(w, s2, b2), out + item);
 }
 
 // Any shape and any 2-byte alignment: one uint16 (four codes) per lane.
@@ -204,18 +169,6 @@ __global__ __launch_bounds__(256) void decompress_transposed_tile_kernel(
   }
 }
 
-template <int THREADS, int WORDS, int UNROLL, bool NT_LOAD, bool NT_STORE>
-void launch_fast(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
-                 int64_t n_words16, int shift, int64_t max_blocks, hipStream_t stream) {
-  const int64_t n_items = n_words16 / (2 * WORDS);
-  const int64_t per_block = (int64_t)THREADS * UNROLL;
-  int64_t blocks = (n_items + per_block - 1) / per_block;
-  if (max_blocks > 0 && blocks > max_blocks) blocks = max_blocks;
-  decompress_kernel<THREADS, WORDS, UNROLL, NT_LOAD, NT_STORE><<<dim3((unsigned)blocks), dim3(THREADS), 0, stream>>>(
-      reinterpret_cast<const uint32_t *>(packed), reinterpret_cast<const half_t *>(scale),
-      reinterpret_cast<const half_t *>(bias), reinterpret_cast<uint4_t *>(out), n_items, shift);
-}
-
 }  // namespace
 
 int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
@@ -226,7 +179,7 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
     const int64_t words_per_row = n_groups * n_ids;
     // tiles of 128 x 128 with 16-byte accesses throughout
     if (words_per_row % (kFastTile / 4) == 0 && n_ids % 8 == 0 && rows % 8 == 0 && (uintptr_t)packed % 16 == 0 &&
-        (uintptr_t)out % 16 == 0 && option_decompress_variant() != 900) {
+        (uintptr_t)out % 16 == 0) {
       const int64_t gx = words_per_row / (kFastTile / 4), gy = (rows + kFastTile - 1) / kFastTile;
       if (gx > 65535 || gy > 0x7fffffff)
         return fail(GQ_ERR_UNSUPPORTED, "transposed decompress: tensor too large (columns=%lld)", (long long)words_per_row * 4);
@@ -242,60 +195,25 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
         reinterpret_cast<half_t *>(out), rows, words_per_row, n_ids);
     return check_launch("decompress_transposed_kernel");
   }
-  const uintptr_t pa = (uintptr_t)packed, oa = (uintptr_t)out;
-  const bool out16 = (oa % 16) == 0;
-  const int variant = option_decompress_variant();
-  // 32-bit words per work item: 1 unless a diagnostic variant asks for wider items.  Items must
-  // tile a group (power-of-two count per group so the group index is a shift) and be aligned.
-  auto usable = [&](int words) {
-    if (!out16 || n_ids % (2 * words) != 0 || pa % (4 * words) != 0) return false;
-    const int64_t ipg = n_ids / (2 * words);
-    return (ipg & (ipg - 1)) == 0;
-  };
-  int words = usable(1) ? 1 : 0;
-  if (variant >= 200 && variant < 300 && usable(2)) words = 2;
-  if (variant >= 400 && variant < 500 && usable(4)) words = 4;
+  // the fast kernel needs whole 32-bit words that tile a group (a power-of-two count per group,
+  // so that the group index is a shift), a 4-byte aligned input and a 16-byte aligned output
+  const int64_t words_per_group = n_ids / 2;
+  const bool fast = n_ids % 2 == 0 && (words_per_group & (words_per_group - 1)) == 0 && (uintptr_t)packed % 4 == 0 &&
+                    (uintptr_t)out % 16 == 0;
   if ((n_words + 1) / 2 / kThreads >= (int64_t)1 << 31) return fail(GQ_ERR_UNSUPPORTED, "decompress: tensor too large");
-  if (words == 0) {
+  if (!fast) {
     const int64_t blocks = (n_words + kThreads - 1) / kThreads;
     decompress_scalar_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
         packed, reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
         reinterpret_cast<half_t *>(out), n_words, n_ids);
     return check_launch("decompress_scalar_kernel");
   }
-  const int shift = __builtin_ctzll((unsigned long long)(n_ids / (2 * words)));
-  const int sub = variant % 100;
-#define GQ_ARGS packed, scale, bias, out, n_words, shift
-  if (words == 4) {
-    launch_fast<256, 4, 1, false, false>(GQ_ARGS, 0, stream);
-  } else if (words == 2) {
-    launch_fast<256, 2, 1, false, true>(GQ_ARGS, 0, stream);
-  } else {
-    switch (sub) {
-      case 1: launch_fast<256, 1, 1, false, false>(GQ_ARGS, 0, stream); break;
-      case 2: launch_fast<256, 1, 1, true, false>(GQ_ARGS, 0, stream); break;
-      case 3: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-      case 4: launch_fast<256, 1, 1, true, true>(GQ_ARGS, 0, stream); break;
-      case 5: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-      case 6: launch_fast<1024, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-      case 7: launch_fast<128, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-      case 8: launch_fast<64, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-      case 9: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
-      case 10: launch_fast<256, 1, 4, false, true>(GQ_ARGS, 0, stream); break;
-      case 11: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 8, stream); break;
-      case 12: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 16, stream); break;
-      case 13: launch_fast<256, 1, 1, false, true>(GQ_ARGS, 256 * 32, stream); break;
-      case 14: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 256 * 4, stream); break;
-      case 15: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 256 * 8, stream); break;
-      case 16: launch_fast<1024, 1, 1, false, true>(GQ_ARGS, 256 * 2, stream); break;
-      case 17: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 256 * 8, stream); break;
-      case 18: launch_fast<256, 1, 2, false, true>(GQ_ARGS, 256 * 16, stream); break;
-      case 19: launch_fast<512, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
-      case 20: launch_fast<128, 1, 2, false, true>(GQ_ARGS, 0, stream); break;
-      default: launch_fast<512, 1, 1, false, true>(GQ_ARGS, 0, stream); break;
-    }
-  }
-#undef GQ_ARGS
+  const int shift = __builtin_ctzll((unsigned long long)words_per_group);
+  const int64_t n_items = n_words / 2;
+  const int64_t blocks = (n_items + kFastThreads - 1) / kFastThreads;
+  decompress_kernel<<<dim3((unsigned)blocks), dim3(kFastThreads), 0, stream>>>(
+      reinterpret_cast<const uint32_t *>(packed), reinterpret_cast<const half_t *>(scale),
+      reinterpret_cast<const half_t *>(bias), reinterpret_cast<uint4_t *>(out), n_items, shift);
   return check_launch("decompress_kernel");
 }
 

@@ -572,27 +572,19 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % BK == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
-  if (!fast_ok || option_gemm_variant() == 1)
+  if (!fast_ok)
     return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
-  const int variant = option_gemm_variant();
 #define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...) \
   launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
-  if (variant != 2 && (k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    int shape = m_rows >= 1024 ? 0 : (m_rows >= 256 ? 1 : 6);
-    if (variant >= 30 && variant <= 36) shape = variant - 30;
-    // the K-split shapes need the K tiles to divide between the groups (and the scale / bias dwords, two groups each)
-    if (shape == 6 && k_in % 256 != 0) shape = 5;
-    switch (shape) {
-      case 6: return GQ_PIPE2(2, 2, 2, 1, 3, 1, 2);  // 128 x 64, 2 x 4 waves splitting K
-      case 0: return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
-      case 1: return GQ_PIPE2(1, 4, 8, 1, 3, 1);  // 256 x 128, 4 waves of 256 x 32
-      case 2: return GQ_PIPE2(1, 4, 4, 1, 3, 2);  // 128 x 128, 4 waves of 128 x 32, two workgroups per CU
-      case 3: return GQ_PIPE2(1, 4, 4, 2, 3, 2);  // 128 x 256, 4 waves of 128 x 64, two workgroups per CU
-      case 4: return GQ_PIPE2(2, 2, 4, 2, 3, 1);  // 256 x 128, 4 waves of 128 x 64
-      default: return GQ_PIPE2(2, 2, 2, 1, 3, 2);  // 128 x 64, 4 waves of 64 x 32: a workgroup on every compute unit at n_out = 16384
-    }
+  if ((k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
+    if (m_rows >= 1024) return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
+    if (m_rows >= 256) return GQ_PIPE2(1, 4, 8, 1, 3, 1);   // 256 x 128, 4 waves of 256 x 32
+    // 128 x 64 (a workgroup on every compute unit at n_out = 16384), 4 waves of 64 x 32; two such
+    // groups of waves split K when the K tiles divide between them (and the scale / bias dwords)
+    if (k_in % 256 == 0) return GQ_PIPE2(2, 2, 2, 1, 3, 1, 2);
+    return GQ_PIPE2(2, 2, 2, 1, 3, 2);
   }
 #undef GQ_PIPE2
   const dim3 grid((unsigned)((n_out + BN - 1) / BN), (unsigned)((m_rows + BM - 1) / BM));

@@ -207,13 +207,12 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream) {
-  const int variant = option_gemv_variant();
   // Large weights at small batches go through the persistent kernel as a sequence of one: its
   // pipelined rings beat the one-shot kernel below once the weight is tens of megabytes (measured:
   // 16384x4096 at one row 14.5 -> 11.7 us). With 3 or 4 rows that holds only for the wide outputs
-  // (4096x16384: 17.2 us one-shot, 18.0 us streamed). Variant 4 forces the route, 2 forbids it.
+  // (4096x16384: 17.2 us one-shot, 18.0 us streamed).
   const bool large = n_out * k_in >= ((int64_t)24 << 20) && (m_rows <= 2 || n_out >= 8192);
-  if ((variant == 4 || (variant == 0 && large)) && m_rows <= 4) {
+  if (large && m_rows <= 4) {
     const int rc =
         launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
     if (rc != GQ_ERR_UNSUPPORTED) return rc;
@@ -221,15 +220,19 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
-  if (fast_ok && variant != 1) {
+  if (fast_ok) {
     const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
     const int64_t row_blocks = (n_out + 15) / 16;
     const bool full = k_in % 512 == 0;
     // rows per wave: reuse the permuted x fragments as often as the row count allows while still
     // filling 256 compute units
-    int r = row_blocks >= 1024 ? 4 : (row_blocks >= 512 ? 2 : 1);
-    if (variant >= 10 && variant < 20) r = variant == 11 ? 1 : (variant == 12 ? 2 : 4);
-    const int gs_mode = (group_size == 64 && full) ? 64 : ((group_size == 128 && full) ? 128 : 0);
+    const int r = row_blocks >= 1024 ? 4 : (row_blocks >= 512 ? 2 : 1);
+    // the GS == 64 / 128 instantiations fetch a chunk's scales and biases as one 16 / 8-byte load per
+    // row: that needs the arrays aligned accordingly; otherwise the 2-byte loads of GS == 0 serve
+    const uintptr_t sb_align = (uintptr_t)scale | (uintptr_t)bias;
+    const int gs_mode = (group_size == 64 && full && sb_align % 16 == 0)
+                            ? 64
+                            : ((group_size == 128 && full && sb_align % 8 == 0) ? 128 : 0);
     const unsigned blocks = (unsigned)((row_blocks + r - 1) / r);
 #define GQ_GEMV_ARGS                                                                                      \
   reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \

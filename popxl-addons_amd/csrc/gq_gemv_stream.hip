@@ -42,10 +42,12 @@ constexpr int kItemOps = 6;             // direct-to-LDS loads per item: 4 packe
 // row blocks per pass (a wave holds their running sums in registers and re-uses the x operands
 // for them); the variant for 4 batch rows has fewer registers to spare
 constexpr int pass_rows(int mc) { return mc == 2 ? 4 : 2; }
-constexpr unsigned kSpinLimit = 1u << 18;
+constexpr unsigned kDefaultSpinLimit = 1u << 18;  // polls without progress before a poller gives up
 constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, batch row)
 
-// Progress of the running sequence on this device.  Every workgroup publishes the number of
+// Progress of a running sequence: a block of words in device memory that the caller provides per
+// sequence (gq_gemv_sequence_ws_f16) or that the library keeps per device (gq_gemv_sequence_f16: one
+// sequence at a time).  Every workgroup publishes the number of
 // entries it has completed in its own word (plain device-scope stores: 256 read-modify-writes of
 // one counter per entry would serialise at the memory side); the last workgroup to leave the
 // kernel clears the words.  Each word has a 128-byte line to itself: with 32 words to a line every
@@ -58,9 +60,12 @@ constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, 
 // without rows of its own loses more to the uneven split of the row blocks than it gains).
 constexpr int kMaxGroups = 256;  // (the watcher keeps a copy of every progress word in LDS)
 constexpr int kProgressStride = 32;  // words
-__device__ __attribute__((aligned(128))) unsigned int g_progress[kMaxGroups * kProgressStride];
-__device__ __attribute__((aligned(128))) unsigned int g_announced[kProgressStride];
-__device__ unsigned int g_exited;  // workgroups that left the kernel
+// layout of the block: [kMaxGroups] progress lines, the watcher's announcement, the count of
+// workgroups that have left the kernel (a line each); all zero between launches
+constexpr int kAnnouncedWord = kMaxGroups * kProgressStride;
+constexpr int kExitedWord = kAnnouncedWord + kProgressStride;
+constexpr int kSequenceWords = kExitedWord + kProgressStride;
+__device__ __attribute__((aligned(256))) unsigned int g_sequence_words[kSequenceWords];
 
 struct Entry {  // = gq_gemv_desc
   const half_t *x;
@@ -170,7 +175,8 @@ __device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint3
 // SINGLE: the sequence is the one entry `single`, passed by value (no descriptor in memory).
 template <int MC, int NS, bool SINGLE>
 __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries, int first_entry,
-                                                 int *__restrict__ status, const Entry single) {
+                                                 int *__restrict__ status, unsigned *__restrict__ words,
+                                                 unsigned spin_limit, const Entry single) {
   static_assert(MC == 2 || MC == 4, "batch capacity");
   constexpr int PR = pass_rows(MC);
   extern __shared__ __attribute__((aligned(64))) char lds[];
@@ -181,6 +187,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   const int wave = uni(tid >> 6);
   const int r = lane & 15, kc = lane >> 4;
   const int G = gridDim.x, b = blockIdx.x;
+  unsigned *const g_progress = words, *const g_announced = words + kAnnouncedWord, *const g_exited = words + kExitedWord;
   CachedEntry *cache = reinterpret_cast<CachedEntry *>(lds + kWaves * kWaveBytes);
   float *mail = reinterpret_cast<float *>(lds + kWaves * kWaveBytes + kMaxEntries * 64);
   Control *ctl = reinterpret_cast<Control *>(mail + 2 * kWaves * kMailFloats);  // two sets of mailboxes
@@ -296,7 +303,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       }
       if (advanced) {
         spins = 0;
-      } else if (++spins > kSpinLimit) {  // some workgroup is not running: give up, let everybody finish
+      } else if (++spins > spin_limit) {  // some workgroup is not running: give up, let everybody finish
         if (lane == 0) {
           __hip_atomic_store(&ctl->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           if (status) atomicExch(status, 1);
@@ -353,13 +360,13 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     // the last workgroup out clears the progress words: by then every poller has seen all it needs
     wait_vm<0>();  // this workgroup's last progress word is in memory before it counts itself out
     unsigned last = 0;
-    if (lane == 0) last = atomicAdd(&g_exited, 1u) == (unsigned)G - 1;
+    if (lane == 0) last = atomicAdd(g_exited, 1u) == (unsigned)G - 1;
     if (uni((int)last)) {
       wait_vm<0>();
       for (int i = lane; i < G; i += 64)
         __hip_atomic_store(&g_progress[i * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(g_announced, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (lane == 0) __hip_atomic_store(&g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     return;
   }
@@ -749,8 +756,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
 
 // (external linkage: the host takes its address for hipFuncSetAttribute)
 template <int MC, int NS>
-__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int first_entry, int *status) {
-  gemv_stream_body<MC, NS, false>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status, Entry{});
+__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int first_entry, int *status,
+                                                                  unsigned *words, unsigned spin_limit) {
+  gemv_stream_body<MC, NS, false>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status, words, spin_limit,
+                                  Entry{});
 }
 
 // one GEMV through the same body: what gq_gemv_f16 launches for large weights
@@ -769,7 +778,7 @@ __global__ __launch_bounds__(kThreadsAll) void gemv_stream_single_kernel(const g
   e.group_size = desc.group_size;
   e.wait_entries = 0;
   e.activation = desc.activation;
-  gemv_stream_body<MC, NS, true>(nullptr, 1, 0, nullptr, e);
+  gemv_stream_body<MC, NS, true>(nullptr, 1, 0, nullptr, nullptr, 0u, e);  // (an entry without a wait touches no progress word)
 }
 
 namespace {
@@ -852,15 +861,17 @@ int launch_gemv_streamed(const uint16_t *x, int64_t m_rows, const uint16_t *pack
   return check_launch("gemv_stream_single_kernel");
 }
 
+int64_t gemv_sequence_workspace_bytes() { return (int64_t)kSequenceWords * 4; }
+
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
-                         hipStream_t stream) {
+                         void *workspace, int64_t spin_limit, hipStream_t stream) {
   int max_m = 1;
   bool supported = count <= (1 << 20);
   for (int64_t i = 0; i < count && supported; ++i) {
     if (host[i].m_rows > max_m) max_m = host[i].m_rows;
     supported = stream_shape_ok(host[i]);
   }
-  if (!supported || option_gemv_variant() == 3) {
+  if (!supported) {
     // any other shape: one launch per entry; stream order provides every dependency
     for (int64_t i = 0; i < count; ++i)
       if (prepacked(host[i]))
@@ -879,6 +890,19 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   int dev = 0;
   const int grid = stream_grid(&dev);
   if (grid == 0) return GQ_ERR_NO_DEVICE;
+  unsigned *words = static_cast<unsigned *>(workspace);
+  if (!words) {
+    // the library's own block of this device (its address differs from device to device)
+    static unsigned *own[kMaxDevices] = {nullptr};
+    if (!own[dev]) {
+      void *ptr = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sequence_words));
+      if (e != hipSuccess || !ptr) return fail((int)e, "hipGetSymbolAddress(progress words): %s", hipGetErrorString(e));
+      own[dev] = static_cast<unsigned *>(ptr);
+    }
+    words = own[dev];
+  }
+  const unsigned spins = spin_limit > 0 ? (unsigned)(spin_limit < 0x7fffffff ? spin_limit : 0x7fffffff) : kDefaultSpinLimit;
 #define GQ_STREAM(MC, NS)                                                                                     \
   do {                                                                                                        \
     constexpr int lds_bytes = stream_lds_bytes<MC, NS>();                                                     \
@@ -893,7 +917,8 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     }                                                                                                         \
     for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
       const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
-      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, (int)first, status);      \
+      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, (int)first, status,       \
+                                                                 words, spins);                               \
     }                                                                                                         \
   } while (0)
   if (max_m <= 2) GQ_STREAM(2, 3);

@@ -1,0 +1,400 @@
+// Fused int4 dequant + matmul for weights grouped along the OUTPUT features, for gfx950:
+// the layout of LinearGQ with dim = -1 or 1, the constructor default of the reference
+// (popxl_addons/layers/linear_gq.py:26, 59-62, 99-101).
+//
+//   packed [k_in, n_out / gs, gs / 4] uint16, scale / bias [k_in, n_out / gs]
+//   W[k][n] = code * scale[k][n / gs] + bias[k][n / gs],   y[m][n] = sum_k x[m][k] * W[k][n] (+ out_bias[n])
+//
+// A packed word holds 8 consecutive OUTPUT features of one input feature k: along the contraction
+// the codes of one output are a weight row (n_out / 2 bytes) apart.  The MFMA wants every lane to
+// hold a run of the contraction index, which this layout cannot give without a transposition, so:
+//
+//  * decode batches (m_rows <= 16), HBM-bound on the packed weight: the MFMA contracts over 4 input
+//    features and the 8 codes of a word at once, with a ONE-HOT B operand that routes code p of a
+//    word to output column p -- see gemv_kn_kernel.  The contraction is split over the waves of a
+//    workgroup (LDS) and over workgroups (fp32 partial sums in a scratch buffer; the last
+//    workgroup to arrive at an output strip adds them up in a fixed order).
+//  * prefill batches: the weight tile is expanded into LDS transposed (gemm_kn_tile_kernel).
+#include "gq_common.h"
+#include "gq_gemv_dequant.h"
+
+namespace gq {
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// Decode kernel.  v_mfma_f32_16x16x32_f16: D[i][c] += sum_{kc, p} A[i][(kc, p)] * B[(kc, p)][c],
+// lane (i = lane % 16, kc = lane / 16) supplies A[i][(kc, 0..7)] and B[(kc, 0..7)][c = lane % 16].
+//   A: lane (i, kc) loads 16 bytes = 4 words = 32 outputs of input feature k0 + kc, at outputs
+//      n_strip + 32 i ..; word t of the lane is the A operand of MFMA t (dequantised, 8 fp16 in the
+//      pair order (0,4,1,5,2,6,3,7) of their positions in the word).
+//   B: column c = (p', mm): position p' of a word, batch row mm of the pair the MFMA serves.
+//      B[(kc, p)][c] = x[mm][k0 + kc] if p == p' else 0 -- one non-zero half per lane.
+//   D_t[i][(p', mm)] = sum_kc W[k0 + kc][n_strip + 32 i + 8 t + order(p')] * x[mm][k0 + kc].
+// One MFMA thus does 4 x 128 x 2 useful multiply-adds of its 8192: the matrix pipe has the room
+// (HBM delivers ~12 bytes per clock to a compute unit, 64 lanes x 16 bytes feed 4 MFMAs per batch
+// pair), and the weights go from memory to the MFMA without a shuffle or an LDS round trip.
+// A wave covers a strip of 512 outputs (256 contiguous bytes per weight row, four rows per load
+// instruction); the 8 waves of a workgroup take every 8th block of 4 input features of the
+// workgroup's K slab.
+// ---------------------------------------------------------------------------------------
+constexpr int kStrip = 512;       // outputs per workgroup
+constexpr int kMaxStrips = 4096;  // arrival counters at the start of the scratch buffer (16 KiB)
+constexpr int kKnWaves = 8;
+constexpr int kKnThreads = kKnWaves * 64;
+
+__device__ __forceinline__ float load_coherent(const float *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_coherent(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// MP: batch-row pairs (m_rows <= 2 MP).  Scratch: one arrival counter per strip (zero before and
+// after every launch) and partial[split][m][n] fp32.
+template <int MP>
+__global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__restrict__ x, int m_rows,
+                                                             const char *__restrict__ packed,
+                                                             const half_t *__restrict__ scale,
+                                                             const half_t *__restrict__ bias,
+                                                             const half_t *__restrict__ out_bias, half_t *__restrict__ y,
+                                                             int n_out, int k_in, int gs_shift, int act, int slab,
+                                                             float *__restrict__ partial, unsigned *__restrict__ counters) {
+  __shared__ float4_t red[kKnWaves][4][64];
+  __shared__ unsigned arrived;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane & 15, kc = lane >> 4;
+  const int strip = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
+  const int n_groups = n_out >> gs_shift;
+  const int64_t row_bytes = n_out >> 1;
+  // this lane's 32 outputs; lanes past n_out re-read the last 16 bytes of the row (results dropped)
+  const int n_lane = strip * kStrip + 32 * i;
+  const int n_load = min(n_lane, n_out - 32);
+  const int g_lane = n_load >> gs_shift;
+  const int k_begin = split * slab, k_end = min(k_in, k_begin + slab);
+
+  // B operand masks: column c = 2 p' + mm keeps x at position p' of the half8
+  const int c = lane & 15, p_sel = c >> 1, mm = c & 1;
+  uint32_t mask[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) mask[r] = (p_sel >> 1) == r ? ((p_sel & 1) ? 0xFFFF0000u : 0x0000FFFFu) : 0u;
+
+  float4_t acc[MP][4];
+#pragma unroll
+  for (int mp = 0; mp < MP; ++mp)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[mp][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  // U blocks of 4 input features per iteration, every load of them issued before the first use:
+  // a wave keeps U KiB of weights in flight
+  constexpr int U = MP <= 2 ? 4 : 2;
+  for (int kb = k_begin + 4 * wave; kb < k_end; kb += 4 * kKnWaves * U) {
+    uint4_t wq[U];
+    uint32_t sv[U], bv[U], xv[U][MP];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = kb + 4 * kKnWaves * u + kc;
+      const bool live = k < k_end;
+      const int kk = live ? k : k_end - 1;  // (past the slab: any valid row, multiplied by x = 0)
+      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(packed + kk * row_bytes + (n_load >> 1)));
+      sv[u] = __builtin_bit_cast(uint16_t, scale[(int64_t)kk * n_groups + g_lane]);
+      bv[u] = __builtin_bit_cast(uint16_t, bias[(int64_t)kk * n_groups + g_lane]);
+#pragma unroll
+      for (int mp = 0; mp < MP; ++mp) {
+        const int m = 2 * mp + mm;
+        xv[u][mp] = (live && m < m_rows) ? (uint32_t)__builtin_bit_cast(uint16_t, x[(int64_t)m * k_in + k]) : 0u;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const half2_t s2 = as_half2(sv[u] | (sv[u] << 16)), b2 = as_half2(bv[u] | (bv[u] << 16));
+      half8_t a[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) a[t] = dequant_word(wq[u][t], s2, b2);
+#pragma unroll
+      for (int mp = 0; mp < MP; ++mp) {
+        const uint32_t xx = xv[u][mp] | (xv[u][mp] << 16);
+        uint4_t bq;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bq[r] = xx & mask[r];
+        const half8_t b = __builtin_bit_cast(half8_t, bq);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[mp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t], b, acc[mp][t], 0, 0, 0);
+      }
+    }
+  }
+
+  // lane (c, rg) of accumulator (mp, t) holds, in element e, row i = 4 rg + e: the output
+  // n = strip + 32 i + 8 t + order(p'), batch row m = 2 mp + mm.  The waves' sums meet in LDS, one
+  // batch-row pair at a time.
+  const bool direct = n_splits == 1;
+#pragma unroll
+  for (int mp = 0; mp < MP; ++mp) {
+    if (mp > 0) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) red[wave][t][lane] = acc[mp][t];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      const int l = threadIdx.x & 63, t = threadIdx.x >> 6;
+      float4_t sum = red[0][t][l];
+#pragma unroll
+      for (int w = 1; w < kKnWaves; ++w) sum += red[w][t][l];
+      const int cc = l & 15, rg = l >> 4;
+      const int m = 2 * mp + (cc & 1);
+      if (m < m_rows) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = strip * kStrip + 32 * (4 * rg + e) + 8 * t + (cc >> 2) + 4 * ((cc >> 1) & 1);  // position p' = cc / 2 holds element p' / 2 + 4 (p' % 2)
+          if (n >= n_out) continue;
+          if (direct) {
+            float v = sum[e];
+            if (out_bias) v += (float)out_bias[n];
+            y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
+          } else {
+            store_coherent(partial + ((int64_t)split * m_rows + m) * n_out + n, sum[e]);
+          }
+        }
+      }
+    }
+  }
+  if (direct) return;
+  // the workgroup's partial sums are in memory before it counts itself in
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned before = __hip_atomic_fetch_add(counters + strip, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = before;
+    if (before == (unsigned)n_splits - 1)  // the last one: leave the counter at zero for the next launch
+      __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (arrived != (unsigned)n_splits - 1) return;
+  // last workgroup of the strip: add the splits in order (the same result whoever arrives last)
+  const int n_strip = min(kStrip, n_out - strip * kStrip);
+  for (int o = threadIdx.x; o < m_rows * n_strip; o += kKnThreads) {
+    const int m = o / n_strip, n = strip * kStrip + o % n_strip;
+    float v = 0.f;
+    for (int s = 0; s < n_splits; ++s) v += load_coherent(partial + ((int64_t)s * m_rows + m) * n_out + n);
+    if (out_bias) v += (float)out_bias[n];
+    y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
+  }
+}
+
+// Any group_size % 4 == 0, any n_out % 4 == 0: one thread per output, up to 16 batch rows per launch;
+// the weight is rebuilt with the two fp16 roundings of the standalone decompress.
+__global__ __launch_bounds__(256) void linear_kn_generic_kernel(const half_t *__restrict__ x, int m_rows,
+                                                                const uint16_t *__restrict__ packed,
+                                                                const half_t *__restrict__ scale,
+                                                                const half_t *__restrict__ bias,
+                                                                const half_t *__restrict__ out_bias, half_t *__restrict__ y,
+                                                                int n_out, int k_in, int group_size, int act) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= n_out) return;
+  const int words = n_out >> 2, n_groups = n_out / group_size;
+  const int shift = 12 - 4 * (n & 3), g = n / group_size;
+  float acc[16];
+#pragma unroll
+  for (int m = 0; m < 16; ++m) acc[m] = 0.f;
+  for (int k = 0; k < k_in; ++k) {
+    const uint32_t w = packed[(int64_t)k * words + (n >> 2)];
+    const half_t code = (half_t)(float)((w >> shift) & 15u);
+    const half_t prod = code * scale[(int64_t)k * n_groups + g];
+    const float wv = (float)(half_t)(prod + bias[(int64_t)k * n_groups + g]);
+#pragma unroll
+    for (int m = 0; m < 16; ++m)
+      if (m < m_rows) acc[m] += (float)x[(int64_t)m * k_in + k] * wv;
+  }
+#pragma unroll
+  for (int m = 0; m < 16; ++m)
+    if (m < m_rows) {
+      float v = acc[m];
+      if (out_bias) v += (float)out_bias[n];
+      y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Prefill kernel.  Workgroup = 4 waves (2 x 2), tile 128 (m) x 128 (n) x 64 (k), as the tile kernel
+// of the other layout, except for how the weight tile reaches LDS: thread (input feature kr = tid
+// % 64, quarter q = tid / 64) loads the 16 bytes = 32 outputs n0 + 32 q .. of feature k0 + kr,
+// expands them and stores them TRANSPOSED, Bs[n][kr]; the 64 lanes of a wave write 128 contiguous
+// bytes of one Bs row per instruction.
+// ---------------------------------------------------------------------------------------
+constexpr int BM = 128, BN = 128, BK = 64, LDK = BK + 8;
+
+__device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
+
+__global__ __launch_bounds__(256) void gemm_kn_tile_kernel(const half_t *__restrict__ x, int m_rows,
+                                                           const char *__restrict__ packed, const half_t *__restrict__ scale,
+                                                           const half_t *__restrict__ bias,
+                                                           const half_t *__restrict__ out_bias, half_t *__restrict__ y,
+                                                           int n_out, int k_in, int gs_shift, int act) {
+  __shared__ __attribute__((aligned(16))) half_t As[BM][LDK];
+  __shared__ __attribute__((aligned(16))) half_t Bs[BN][LDK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int n_groups = n_out >> gs_shift;
+  const int64_t row_bytes = n_out >> 1;
+
+  const int a_col = (tid & 7) * 8, a_row = tid >> 3;
+  const half_t *a_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a_src[i] = x + (int64_t)min(m0 + a_row + 32 * i, m_rows - 1) * k_in + a_col;
+  const int kr = tid & 63, q = tid >> 6;
+  const int n_load = min(n0 + 32 * q, n_out - 32);  // columns past n_out re-read the last 32 (never stored to y)
+  const int g = n_load >> gs_shift;
+  const char *b_src = packed + (n_load >> 1);
+
+  float16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  uint4_t a_reg[4], b_reg;
+  half_t s_reg, z_reg;
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a_reg[i] = *reinterpret_cast<const uint4_t *>(a_src[i] + k0);
+    b_reg = *reinterpret_cast<const uint4_t *>(b_src + (int64_t)(k0 + kr) * row_bytes);
+    s_reg = scale[(int64_t)(k0 + kr) * n_groups + g];
+    z_reg = bias[(int64_t)(k0 + kr) * n_groups + g];
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4_t *>(&As[a_row + 32 * i][a_col]) = a_reg[i];
+    const half2_t s2 = {s_reg, s_reg}, z2 = {z_reg, z_reg};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      // pair order (0,4) (1,5) (2,6) (3,7) of the word's eight outputs
+      const half8_t v = dequant_word(b_reg[w], s2, z2);
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        Bs[32 * q + 8 * w + p][kr] = v[2 * p];
+        Bs[32 * q + 8 * w + p + 4][kr] = v[2 * p + 1];
+      }
+    }
+  };
+
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+  load_tile(0);
+  for (int k0 = 0; k0 < k_in; k0 += BK) {
+    __syncthreads();
+    store_tile();
+    __syncthreads();
+    if (k0 + BK < k_in) load_tile(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      half8_t a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const half8_t *>(&As[wm * 64 + i * 32 + frag_row][ks + frag_k]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const half8_t *>(&Bs[wn * 64 + j * 32 + frag_row][ks + frag_k]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // D[m][n]: lane holds n = lane % 32 and m = 8 * (e / 4) + 4 * (lane / 32) + e % 4
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+      if (n >= n_out) continue;
+      const float ob = out_bias ? (float)out_bias[n] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)apply_activation(acc[i][j][e] + ob, act);
+      }
+    }
+}
+
+// K slabs of the decode kernel: enough workgroups to fill the device twice over, slabs a multiple
+// of the 32 input features that the 8 waves take per round
+int kn_splits(int64_t n_out, int64_t k_in, int64_t *slab_out) {
+  const int64_t strips = (n_out + kStrip - 1) / kStrip;
+  int64_t splits = (512 + strips - 1) / strips;  // two workgroups per compute unit
+  const int64_t max_splits = (k_in + 127) / 128;  // at least four rounds per wave
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 64) splits = 64;
+  if (splits < 1) splits = 1;
+  int64_t slab = (k_in + splits - 1) / splits;
+  slab = (slab + 31) / 32 * 32;
+  splits = (k_in + slab - 1) / slab;
+  *slab_out = slab;
+  return (int)splits;
+}
+
+bool kn_fast_shape(const uint16_t *x, const uint16_t *packed, int64_t n_out, int64_t k_in, int64_t group_size) {
+  const bool pow2 = (group_size & (group_size - 1)) == 0;
+  return pow2 && group_size >= 32 && n_out % 32 == 0 && n_out >= 32 && n_out <= (int64_t)kMaxStrips * kStrip &&
+         k_in > 0 && ((uintptr_t)packed % 16) == 0 && ((uintptr_t)x % 2) == 0;
+}
+
+}  // namespace
+
+// Scratch bytes the decode kernel needs for this problem (0: none): the arrival counters (a fixed
+// 16 KiB at the start, so that calls of any shape find them at the same place), then fp32 partial
+// sums per K slab.
+int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (m_rows < 1 || m_rows > 16 || k_in < 1) return 0;
+  const bool pow2 = (group_size & (group_size - 1)) == 0;
+  if (!pow2 || group_size < 32 || n_out % 32 != 0 || n_out < 32 || n_out > (int64_t)kMaxStrips * kStrip) return 0;
+  int64_t slab = 0;
+  const int splits = kn_splits(n_out, k_in, &slab);
+  if (splits == 1) return 0;
+  return (int64_t)kMaxStrips * 4 + splits * m_rows * n_out * 4;
+}
+
+// `workspace`: linear_kn_workspace_bytes() bytes of device memory whose first 16 KiB (the counters)
+// are zero; the kernel leaves them zero.
+int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                     const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                     int64_t group_size, int act, void *workspace, hipStream_t stream) {
+  const half_t *xh = reinterpret_cast<const half_t *>(x), *sh = reinterpret_cast<const half_t *>(scale),
+               *bh = reinterpret_cast<const half_t *>(bias), *oh = reinterpret_cast<const half_t *>(out_bias);
+  half_t *yh = reinterpret_cast<half_t *>(y);
+  const bool fast = kn_fast_shape(x, packed, n_out, k_in, group_size);
+  const int gs_shift = fast ? __builtin_ctzll((unsigned long long)group_size) : 0;
+  if (fast && m_rows <= 16) {
+    int64_t slab = 0;
+    const int splits = kn_splits(n_out, k_in, &slab);
+    const int64_t strips = (n_out + kStrip - 1) / kStrip;
+    unsigned *counters = static_cast<unsigned *>(workspace);
+    float *partial = reinterpret_cast<float *>(counters + kMaxStrips);
+    const dim3 grid((unsigned)strips, (unsigned)splits), block(kKnThreads);
+#define GQ_KN(MP)                                                                                                    \
+  gemv_kn_kernel<MP><<<grid, block, 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, oh, yh, \
+                                                 (int)n_out, (int)k_in, gs_shift, act, (int)slab, partial, counters)
+    if (m_rows <= 2) GQ_KN(1);
+    else if (m_rows <= 4) GQ_KN(2);
+    else if (m_rows <= 8) GQ_KN(4);
+    else GQ_KN(8);
+#undef GQ_KN
+    return check_launch("gemv_kn_kernel");
+  }
+  if (fast && k_in % BK == 0 && ((uintptr_t)x % 16) == 0) {
+    const dim3 grid((unsigned)((n_out + BN - 1) / BN), (unsigned)((m_rows + BM - 1) / BM));
+    if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_linear_kn: m_rows=%lld too large", (long long)m_rows);
+    gemm_kn_tile_kernel<<<grid, dim3(256), 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, oh,
+                                                        yh, (int)n_out, (int)k_in, gs_shift, act);
+    return check_launch("gemm_kn_tile_kernel");
+  }
+  const unsigned blocks = (unsigned)((n_out + 255) / 256);
+  for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
+    const int m = (int)(m_rows - m0 < 16 ? m_rows - m0 : 16);
+    linear_kn_generic_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(xh + m0 * k_in, m, packed, sh, bh, oh, yh + m0 * n_out,
+                                                                     (int)n_out, (int)k_in, (int)group_size, act);
+  }
+  return check_launch("linear_kn_generic_kernel");
+}
+
+}  // namespace gq

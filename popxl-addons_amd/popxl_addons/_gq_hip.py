@@ -10,7 +10,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _DEFAULT_LIB = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libgq_hip.so")
 
-GQ_ABI_VERSION = 1
+GQ_ABI_VERSION = 2
 GQ_ERR_NULL_POINTER = -1
 GQ_ERR_BAD_SHAPE = -2
 GQ_ERR_MISALIGNED = -3
@@ -33,17 +33,21 @@ def activation_code(activation):
 EXPORTS = (
     "gq_abi_version",
     "gq_last_error",
-    "gq_set_option",
     "gq_decompress_f16",
     "gq_decompress_f16_transposed",
     "gq_gemv_f16",
     "gq_gemm_f16",
     "gq_linear_f16",
     "gq_linear_act_f16",
+    "gq_linear_kn_workspace_bytes",
+    "gq_linear_kn_act_f16",
     "gq_gemv_sequence_f16",
+    "gq_gemv_sequence_workspace_bytes",
+    "gq_gemv_sequence_ws_f16",
     "gq_gemv_prepacked_bytes",
     "gq_gemv_prepack_f16",
     "gq_compress_f16",
+    "gq_compress_f32",
 )
 
 
@@ -80,8 +84,6 @@ def load():
     lib.gq_abi_version.restype = ctypes.c_int
     lib.gq_last_error.argtypes = []
     lib.gq_last_error.restype = ctypes.c_char_p
-    lib.gq_set_option.argtypes = [ctypes.c_char_p, i64]
-    lib.gq_set_option.restype = ctypes.c_int
     for name in ("gq_decompress_f16", "gq_decompress_f16_transposed"):
         fn = getattr(lib, name)
         fn.argtypes = [p, p, p, p, i64, i64, i64, p]
@@ -92,14 +94,24 @@ def load():
         fn.restype = ctypes.c_int
     lib.gq_linear_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p]
     lib.gq_linear_act_f16.restype = ctypes.c_int
+    lib.gq_linear_kn_workspace_bytes.argtypes = [i64, i64, i64, i64]
+    lib.gq_linear_kn_workspace_bytes.restype = i64
+    lib.gq_linear_kn_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
+    lib.gq_linear_kn_act_f16.restype = ctypes.c_int
     lib.gq_gemv_sequence_f16.argtypes = [p, p, i64, p, p]
     lib.gq_gemv_sequence_f16.restype = ctypes.c_int
+    lib.gq_gemv_sequence_workspace_bytes.argtypes = []
+    lib.gq_gemv_sequence_workspace_bytes.restype = i64
+    lib.gq_gemv_sequence_ws_f16.argtypes = [p, p, i64, p, p, i64, i64, p]
+    lib.gq_gemv_sequence_ws_f16.restype = ctypes.c_int
     lib.gq_gemv_prepacked_bytes.argtypes = [i64, i64, i64]
     lib.gq_gemv_prepacked_bytes.restype = i64
     lib.gq_gemv_prepack_f16.argtypes = [p, p, p, p, i64, i64, i64, p]
     lib.gq_gemv_prepack_f16.restype = ctypes.c_int
-    lib.gq_compress_f16.argtypes = [p, p, p, p, p, i64, i64, i64, p]
-    lib.gq_compress_f16.restype = ctypes.c_int
+    for name in ("gq_compress_f16", "gq_compress_f32"):
+        fn = getattr(lib, name)
+        fn.argtypes = [p, p, p, p, p, i64, i64, i64, p]
+        fn.restype = ctypes.c_int
     if lib.gq_abi_version() != GQ_ABI_VERSION:
         raise ImportError(f"{path}: ABI version {lib.gq_abi_version()} != expected {GQ_ABI_VERSION}")
     _lib = lib
@@ -118,8 +130,20 @@ def call(name, *args):
         raise GQHipError(name, rc, lib.gq_last_error().decode("utf-8", "replace"))
 
 
-def set_option(name, value):
-    call("gq_set_option", name.encode(), int(value))
+_kn_workspaces = {}
+
+
+def linear_kn_workspace(device, nbytes):
+    """The scratch buffer of gq_linear_kn_act_f16 on `device` (one per device, grown on demand; its
+    arrival counters start at zero and every call leaves them zero).  Calls that share it are
+    ordered by the stream they are enqueued on: use one stream per device for this layer."""
+    import torch
+
+    ws = _kn_workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _kn_workspaces[device] = ws
+    return ws
 
 
 class PrepackedWeight:
@@ -159,10 +183,17 @@ class GemvSequence:
     sets to 1 if it gave up waiting.
     """
 
-    def __init__(self, device):
+    def __init__(self, device, own_workspace=False, spin_limit=0):
+        """own_workspace: keep the kernel's progress words in a buffer of this object
+        (gq_gemv_sequence_ws_f16) instead of the block the library holds per device, so that
+        several sequences may be enqueued on different streams; spin_limit: polls without
+        progress after which a wait gives up (0: the library's default)."""
         import numpy as np
 
         self.device = device
+        self.own_workspace = own_workspace or spin_limit > 0
+        self.spin_limit = int(spin_limit)
+        self._workspace = None
         self.dtype = np.dtype(
             [("x", "<u8"), ("packed", "<u8"), ("scale", "<u8"), ("bias", "<u8"), ("out_bias", "<u8"), ("y", "<u8"),
              ("m_rows", "<i4"), ("n_out", "<i4"), ("k_in", "<i4"), ("group_size", "<i4"), ("wait_entries", "<i4"),
@@ -219,7 +250,11 @@ class GemvSequence:
         if self._host is None:
             self._finalise()
         call(
-            "gq_gemv_sequence_f16",
+            "gq_linear_kn_workspace_bytes",
+    "gq_linear_kn_act_f16",
+    "gq_gemv_sequence_f16",
+    "gq_gemv_sequence_workspace_bytes",
+    "gq_gemv_sequence_ws_f16",
             self._host.ctypes.data,
             self._dev.data_ptr(),
             len(self.entries),

@@ -7,8 +7,8 @@ import numpy as np
 
 from popxl_addons import _gq_hip
 from popxl_addons.ops.group_quantize_decompress import (
+    group_quantize_compress,
     group_quantize_compress_numpy,
-    group_quantize_decompress,
 )
 from popxl_addons.utils import NamedTensors, Variable, WeightsDict, _numpy_dtype_of
 
@@ -43,8 +43,9 @@ class LinearGQ:
         - replica_grouping: must be None (single GPU, no variable sharding)
         - group_size (int): values per (scale, bias) pair; must be set to a positive multiple of 4
         - dim (int): dimension of the [in, out] weight matrix that is grouped.
-                     0: groups run along the input features (fused dequant-matmul kernels);
+                     0: groups run along the input features;
                      1 or -1: groups run along the output features.
+                     Both layouts run fused dequant-matmul kernels.
         """
         if replica_grouping is not None:
             raise NotImplementedError("LinearGQ here runs on one GPU: replica_grouping must be None")
@@ -103,7 +104,7 @@ class LinearGQ:
         """y = x @ decompress(weight) (+ bias), linear_gq.py:99-109.  x: float16 [..., in] on the GPU.
 
         activation (None, "relu", "gelu_tanh") is an addition to the reference's signature: the
-        epilogue is fused into the kernel for dim=0 and applied by torch otherwise."""
+        epilogue is fused into the kernel."""
         import torch
 
         act = _gq_hip.activation_code(activation)
@@ -121,40 +122,33 @@ class LinearGQ:
             raise ValueError(f"LinearGQ: x has {in_features} features but weight_compressed is {v.weight_compressed.shape}")
         b = v.bias.data if self.bias else None
 
-        if self.dim == 0:
-            x2 = x.reshape(-1, in_features).contiguous()
-            with torch.cuda.device(x.device):
-                y = torch.empty((x2.shape[0], self.out_features), dtype=torch.float16, device=x.device)
-                _gq_hip.call(
-                    "gq_linear_act_f16",
-                    x2.data_ptr(),
-                    x2.shape[0],
-                    v.weight_compressed.data.data_ptr(),
-                    v.weight_decompression_scale.data.data_ptr(),
-                    v.weight_decompression_bias.data.data_ptr(),
-                    0 if b is None else b.data_ptr(),
-                    y.data_ptr(),
-                    self.out_features,
-                    in_features,
-                    self.group_size,
-                    act,
-                    torch.cuda.current_stream(x.device).cuda_stream,
-                )
-            return y.reshape(*x.shape[:-1], self.out_features)
-
-        # groups along the output features: the weight comes out of the decompress kernel as
-        # [in, out] and feeds a dense matmul
-        w = group_quantize_decompress(
-            v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data, self.dim
-        )
-        y = x @ w
-        if b is not None:
-            y = y + b
-        if act == _gq_hip.GQ_ACT_RELU:
-            y = torch.relu(y)
-        elif act == _gq_hip.GQ_ACT_GELU_TANH:
-            y = torch.nn.functional.gelu(y.float(), approximate="tanh").to(y.dtype)
-        return y
+        x2 = x.reshape(-1, in_features).contiguous()
+        m_rows = x2.shape[0]
+        with torch.cuda.device(x.device):
+            y = torch.empty((m_rows, self.out_features), dtype=torch.float16, device=x.device)
+            args = (
+                x2.data_ptr(),
+                m_rows,
+                v.weight_compressed.data.data_ptr(),
+                v.weight_decompression_scale.data.data_ptr(),
+                v.weight_decompression_bias.data.data_ptr(),
+                0 if b is None else b.data_ptr(),
+                y.data_ptr(),
+                self.out_features,
+                in_features,
+                self.group_size,
+                act,
+            )
+            stream = torch.cuda.current_stream(x.device).cuda_stream
+            if self.dim == 0:
+                _gq_hip.call("gq_linear_act_f16", *args, stream)
+            else:
+                # groups along the output features: weight rows are input features
+                need = _gq_hip.load().gq_linear_kn_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)
+                ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None
+                _gq_hip.call("gq_linear_kn_act_f16", *args, 0 if ws is None else ws.data_ptr(),
+                             0 if ws is None else ws.numel(), stream)
+        return y.reshape(*x.shape[:-1], self.out_features)
 
     __call__ = build
 
@@ -164,9 +158,10 @@ class LinearGQ:
     def fuse(cls, layers):
         """One layer computing the concatenated outputs of `layers` (e.g. the Q, K and V projections
         of a decoder block, which read the same activations): y = cat([l(x) for l in layers], -1) in
-        a single kernel pass over x.  Needs groups along the input features (dim=0), where the
-        variables of the layers stack along their first axis; all layers must agree in
-        group_size, bias and input width.  The new layer owns copies of the variables.
+        a single kernel pass over x.  The variables of the layers stack along their first axis for
+        dim=0 (weight rows are output features) and along the group axis for dim=-1 / 1 (weight rows
+        are input features); all layers must agree in dim, group_size, bias and input width.  The
+        new layer owns copies of the variables.
         """
         import torch
 
@@ -177,19 +172,21 @@ class LinearGQ:
         for layer in layers:
             if layer.variables is None:
                 raise ValueError("LinearGQ.fuse: every layer needs its variables (build it or call init_variables)")
-            if layer.dim != 0:
-                raise NotImplementedError("LinearGQ.fuse: only dim=0 layers stack along the output features")
+            if (layer.dim == 0) != (first.dim == 0):
+                raise NotImplementedError("LinearGQ.fuse: layers grouped along different axes do not stack")
             if layer.group_size != first.group_size or layer.bias != first.bias:
                 raise ValueError("LinearGQ.fuse: layers differ in group_size or bias")
-            if layer.variables.weight_compressed.shape[1:] != first.variables.weight_compressed.shape[1:]:
+            mine, theirs = layer.variables.weight_compressed.shape, first.variables.weight_compressed.shape
+            if (mine[1:] != theirs[1:]) if first.dim == 0 else (mine[0] != theirs[0]):
                 raise ValueError("LinearGQ.fuse: layers differ in input features")
-        fused = cls(sum(l.out_features for l in layers), bias=first.bias, group_size=first.group_size, dim=0)
+        fused = cls(sum(l.out_features for l in layers), bias=first.bias, group_size=first.group_size, dim=first.dim)
+        axis = 0 if first.dim == 0 else 1
         names = ["weight_compressed", "weight_decompression_scale", "weight_decompression_bias"]
-        if first.bias:
-            names.append("bias")
         fused.variables = NamedTensors(
-            **{n: Variable(n, torch.cat([l.variables[n].data for l in layers], dim=0).contiguous()) for n in names}
+            **{n: Variable(n, torch.cat([l.variables[n].data for l in layers], dim=axis).contiguous()) for n in names}
         )
+        if first.bias:
+            fused.variables.insert("bias", Variable("bias", torch.cat([l.variables.bias.data for l in layers]).contiguous()))
         return fused
 
     def prepacked(self):
@@ -215,6 +212,12 @@ class LinearGQ:
         import torch
 
         dtype = torch.float32 if dtype is None else dtype
+        weight_t = nn_layer.weight.T.detach()
+        if weight_t.is_cuda:
+            # the packer on the device: the same bits as the numpy function gives for this array
+            compressed = tuple(a.cpu().numpy() for a in group_quantize_compress(weight_t, group_size, dim=dim))
+        else:
+            compressed = group_quantize_compress_numpy(weight_t.numpy(), group_size, dim=dim)
         state_dict = dict(
             zip(
                 (
@@ -222,7 +225,7 @@ class LinearGQ:
                     variables.weight_decompression_scale,
                     variables.weight_decompression_bias,
                 ),
-                group_quantize_compress_numpy(nn_layer.weight.T.detach().cpu().numpy(), group_size, dim=dim),
+                compressed,
             )
         )
         if "bias" in variables.keys():

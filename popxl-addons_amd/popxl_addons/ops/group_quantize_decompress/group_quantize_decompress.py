@@ -122,8 +122,9 @@ def group_quantize_decompress(t, group_scale, group_bias, dim=-1):
 
 def group_quantize_compress(t, group_size: int, dim: int = -1):
     """
-    Device-side compress of a float16 matrix (torch.Tensor on a HIP device): the same
-    (packed, scale, bias) bits as group_quantize_compress_numpy gives for a float16 array.
+    Device-side compress of a float16 or float32 tensor (torch.Tensor on a HIP device): the same
+    (packed, scale, bias) bits as group_quantize_compress_numpy gives for the same array (float32
+    input is quantised in float32 arithmetic, as the reference does at :186-192).
 
     Raises ValueError for non-finite input, like the numpy function (:182-183).
     """
@@ -131,8 +132,8 @@ def group_quantize_compress(t, group_size: int, dim: int = -1):
 
     if not t.is_cuda:
         raise RuntimeError("group_quantize_compress runs on the GPU only")
-    if t.dtype != torch.float16:
-        raise TypeError("group_quantize_compress takes float16 input")
+    if t.dtype not in (torch.float16, torch.float32):
+        raise TypeError("group_quantize_compress takes float16 or float32 input")
     if dim != -1:
         perm = list(range(t.dim()))
         perm.append(perm.pop(dim))
@@ -151,7 +152,7 @@ def group_quantize_compress(t, group_size: int, dim: int = -1):
         bias = torch.empty((*lead, n_groups, 1), dtype=torch.float16, device=t.device)
         flag = torch.zeros(1, dtype=torch.int32, device=t.device)
         _gq_hip.call(
-            "gq_compress_f16",
+            "gq_compress_f16" if t.dtype == torch.float16 else "gq_compress_f32",
             t.data_ptr(),
             packed.data_ptr(),
             scale.data_ptr(),

@@ -42,11 +42,8 @@ def test_exact_rational_vectors(hip, device):
     packed = np.tile(np.array([0x0123, 0x4567, 0x89AB, 0xCDEF], np.uint16), (n, 1, 1))
     scale = z["scale_bits"].view(np.float16).reshape(n, 1, 1)
     bias = z["bias_bits"].view(np.float16).reshape(n, 1, 1)
-    for variant in (0, 1, 201, 401):
-        hip.set_option("decompress_variant", variant)
-        out = _run(packed, scale, bias, device)
-        assert_bits_equal(out, z["expected_bits"].view(np.float16), f"exact vectors, variant {variant}")
-    hip.set_option("decompress_variant", 0)
+    out = _run(packed, scale, bias, device)
+    assert_bits_equal(out, z["expected_bits"].view(np.float16), "exact vectors")
     # same pairs through the 2-byte-per-lane kernel (n_ids odd) and the transposed kernel
     packed3 = np.tile(np.array([0x0123, 0x4567, 0x89AB], np.uint16), (n, 1, 1))
     out = _run(packed3, scale, bias, device)
@@ -86,19 +83,13 @@ def test_ragged_shapes_all_dims(hip, device, oracle, rows, n_groups, n_ids):
 @pytest.mark.parametrize("n_groups,n_ids", [(4, 8), (3, 32), (2, 16), (16, 16), (1, 64)])
 def test_transposed_tile_kernel(hip, device, oracle, rows, n_groups, n_ids):
     """dim=0 through the 128 x 128 tile kernel (columns a multiple of 128, rows a multiple of 8,
-    8 or more uint16 per group): bit-exact, the forced simple kernel gives the same, and nothing
-    is written outside the result."""
+    8 or more uint16 per group): bit-exact, and nothing is written outside the result."""
     rng = np.random.default_rng(rows * 100 + n_groups * 10 + n_ids)
     packed = rng.integers(0, 65536, (rows, n_groups, n_ids), dtype=np.uint16)
     scale = rng.normal(0, 0.01, (rows, n_groups, 1)).astype(np.float16)
     bias = rng.normal(0, 0.1, (rows, n_groups, 1)).astype(np.float16)
     want_t = oracle.c_decompress(packed, scale, bias).T
     assert_bits_equal(_run(packed, scale, bias, device, 0), want_t, "tile kernel")
-    try:
-        hip.set_option("decompress_variant", 900)
-        assert_bits_equal(_run(packed, scale, bias, device, 0), want_t, "simple kernel")
-    finally:
-        hip.set_option("decompress_variant", 0)
     p_dev, s_dev, b_dev = to_dev(packed, device), to_dev(scale, device), to_dev(bias, device)
     buf = torch.full((want_t.size + 128,), 123.0, dtype=torch.float16, device=device)
     hip.call("gq_decompress_f16_transposed", p_dev.data_ptr(), s_dev.data_ptr(), b_dev.data_ptr(), buf.data_ptr() + 128,
@@ -109,18 +100,13 @@ def test_transposed_tile_kernel(hip, device, oracle, rows, n_groups, n_ids):
     assert np.all(res[:64] == 123.0) and np.all(res[64 + want_t.size :] == 123.0), "wrote out of bounds"
 
 
-def test_every_kernel_variant_and_alignment(hip, device, oracle):
+def test_alignment_fallbacks(hip, device, oracle):
     rng = np.random.default_rng(8)
     packed = rng.integers(0, 65536, (67, 9, 16), dtype=np.uint16)
     scale = rng.normal(0, 0.01, (67, 9, 1)).astype(np.float16)
     bias = rng.normal(0, 0.1, (67, 9, 1)).astype(np.float16)
     want = oracle.c_decompress(packed, scale, bias)
-    try:
-        for variant in list(range(0, 21)) + [201, 401]:
-            hip.set_option("decompress_variant", variant)
-            assert_bits_equal(_run(packed, scale, bias, device), want, f"variant {variant}")
-    finally:
-        hip.set_option("decompress_variant", 0)
+    assert_bits_equal(_run(packed, scale, bias, device), want, "aligned")
     # pointers that are only 2-, 4- or 8-byte aligned, and a guarded output buffer
     p_dev, s_dev, b_dev = to_dev(packed, device), to_dev(scale, device), to_dev(bias, device)
     n_out = want.size

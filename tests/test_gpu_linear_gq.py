@@ -84,6 +84,48 @@ def test_device_compress_bit_exact(hip, device, oracle, group_size):
     assert_bits_equal(b.cpu().numpy(), bw, "bias")
 
 
+@pytest.mark.parametrize("group_size", [8, 16, 32, 64, 128, 256, 512, 12, 40])
+def test_device_compress_f32_bit_exact(hip, device, oracle, group_size):
+    """float32 input (what torch_mapping feeds the packer): max / min cast to float16, the quotient
+    in float32 -- the same bits as the C oracle and as the numpy packer on the same array."""
+    rng = np.random.default_rng(100 + group_size)
+    cols = group_size * 7
+    w = rng.normal(0, 0.02, (129, cols)).astype(np.float32)
+    w[rng.random(w.shape) < 1e-2] *= 8
+    w[5, :group_size] = 0.125  # a constant group
+    w[6, : 2 * group_size] = 0.0
+    p, s, b = group_quantize_compress(to_dev(w, device), group_size)
+    torch.cuda.synchronize()
+    pw, sw, bw = oracle.c_compress(w, group_size)
+    # float32 values between two float16 numbers can fall below the float16 minimum of their group:
+    # the reference is undefined there (a negative code); such groups are left out of the comparison
+    pn, sn, bn = group_quantize_compress_numpy(w, group_size)
+    assert_bits_equal(s.cpu().numpy(), sw, "scale")
+    assert_bits_equal(b.cpu().numpy(), bw, "bias")
+    assert np.array_equal(p.cpu().numpy(), pn), "device packer differs from the numpy packer"
+    g = w.reshape(129, 7, group_size)
+    defined = (g >= bw.astype(np.float32)).all(-1) & (np.rint((g - bw.astype(np.float32)) / np.where(sw == 0, 1, sw).astype(np.float32)) <= 15).all(-1)
+    assert defined.mean() > 0.5
+    assert np.array_equal(p.cpu().numpy()[defined], pw[defined])
+
+
+def test_device_compress_f32_full_size_and_nonfinite(hip, device, oracle):
+    """A 4096 x 4096 float32 weight grouped along either axis (the two LinearGQ layouts) equals the
+    numpy packer; NaN raises."""
+    rng = np.random.default_rng(12)
+    w = rng.normal(0, 0.02, (4096, 4096)).astype(np.float32)
+    wd = to_dev(w, device)
+    for dim in (-1, 0):
+        p, s, b = group_quantize_compress(wd, 64, dim=dim)
+        pn, sn, bn = group_quantize_compress_numpy(w, 64, dim=dim)
+        assert np.array_equal(p.cpu().numpy(), pn), dim
+        assert_bits_equal(s.cpu().numpy(), sn, "scale")
+        assert_bits_equal(b.cpu().numpy(), bn, "bias")
+    w[100, 7] = np.inf
+    with pytest.raises(ValueError):
+        group_quantize_compress(to_dev(w, device), 64)
+
+
 def test_device_compress_output_alignment(hip, device, oracle):
     """A packed output that is only 4-byte aligned takes the kernel with 8 elements per lane
     (32-bit stores) instead of 16 (64-bit stores): same bits."""
@@ -216,7 +258,7 @@ def test_fuse_rejects_mismatched_layers(hip, device):
 @pytest.mark.parametrize("dim", [0, -1])
 @pytest.mark.parametrize("activation", ["relu", "gelu_tanh"])
 def test_linear_gq_activation(hip, device, oracle, dim, activation):
-    """LinearGQ.build(x, activation=...): fused epilogue for dim=0, torch epilogue otherwise."""
+    """LinearGQ.build(x, activation=...): the epilogue is fused into the kernel in both layouts."""
     in_features, out_features, group_size = 256, 384, 64
     torch.manual_seed(4)
     nn_layer = torch.nn.Linear(in_features, out_features)

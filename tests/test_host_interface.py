@@ -52,9 +52,40 @@ def test_abi_version_and_error_text_without_gpu():
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_f16", 16, 1, 16, 16, 16, 0, 16, 8, 64, 6, None)  # group_size % 4
     assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    # the [k_in, n_out] layout: its own argument rules and the workspace contract
     with pytest.raises(_gq_hip.GQHipError) as e:
-        _gq_hip.call("gq_set_option", b"no_such_option", 1)
-    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED
+        _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 96, 64, 64, 0, None, 0, None)  # 96 % 64 != 0
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE and "n_out" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 128, 64, 64, 3, None, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "activation" in str(e.value)
+    need = lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 64)
+    assert need > 16384 and need <= 16384 + 64 * 16384 * 4 and need == lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 32)
+    assert lib.gq_linear_kn_workspace_bytes(4, 16384, 4096, 64) == 16384 + (need - 16384) * 4
+    assert lib.gq_linear_kn_workspace_bytes(1, 128, 64, 64) == 0  # one K slab: no scratch
+    assert lib.gq_linear_kn_workspace_bytes(17, 16384, 4096, 64) == 0  # prefill batches need none
+    assert lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 20) == 0  # generic kernel
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 16384, 4096, 64, 0, None, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER and "workspace" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 16384, 4096, 64, 0, 256, need - 1, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE and "workspace" in str(e.value)
+    # the sequence with a caller-owned workspace
+    assert lib.gq_gemv_sequence_workspace_bytes() == (256 + 2) * 128
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_ws_f16", 16, 16, 1, None, None, 0, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER and "workspace" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_gemv_sequence_ws_f16", 16, 16, 1, None, 256, 100, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    # device packer for binary32 input
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_compress_f32", 16, 16, 16, 16, 0, 4, 4, 6, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_compress_f32", 18, 16, 16, 16, 0, 4, 4, 8, None)
+    assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED
     # sequence descriptors are validated on the host copy: an entry cannot wait for itself
     import numpy as np
 
