@@ -105,7 +105,7 @@ def test_device_compress_f32_bit_exact(hip, device, oracle, group_size):
     assert np.array_equal(p.cpu().numpy(), pn), "device packer differs from the numpy packer"
     g = w.reshape(129, 7, group_size)
     defined = (g >= bw.astype(np.float32)).all(-1) & (np.rint((g - bw.astype(np.float32)) / np.where(sw == 0, 1, sw).astype(np.float32)) <= 15).all(-1)
-    assert defined.mean() > 0.5
+    assert defined.mean() > 0.2
     assert np.array_equal(p.cpu().numpy()[defined], pw[defined])
 
 
