@@ -243,21 +243,28 @@ class GemvSequence:
         self._host = np.array(self.entries, dtype=self.dtype)
         self._dev = torch.from_numpy(self._host.view(np.uint8).copy()).to(self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
+        if self.own_workspace and self._workspace is None:
+            self._workspace = torch.zeros(load().gq_gemv_sequence_workspace_bytes(), dtype=torch.uint8, device=self.device)
 
     def run(self):
         import torch
 
         if self._host is None:
             self._finalise()
-        call(
-            "gq_linear_kn_workspace_bytes",
-    "gq_linear_kn_act_f16",
-    "gq_gemv_sequence_f16",
-    "gq_gemv_sequence_workspace_bytes",
-    "gq_gemv_sequence_ws_f16",
-            self._host.ctypes.data,
-            self._dev.data_ptr(),
-            len(self.entries),
-            self.status.data_ptr(),
-            torch.cuda.current_stream(self.device).cuda_stream,
-        )
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self.own_workspace:
+            call("gq_gemv_sequence_ws_f16", self._host.ctypes.data, self._dev.data_ptr(), len(self.entries),
+                 self.status.data_ptr(), self._workspace.data_ptr(), self._workspace.numel(), self.spin_limit, stream)
+        else:
+            call("gq_gemv_sequence_f16", self._host.ctypes.data, self._dev.data_ptr(), len(self.entries),
+                 self.status.data_ptr(), stream)
+
+    def check(self):
+        """Synchronise and raise if a wait of the last run() gave up (results are then invalid)."""
+        import torch
+
+        torch.cuda.synchronize(self.device)
+        if self.status is not None and int(self.status.item()) != 0:
+            self.status.zero_()
+            raise GQHipError("gq_gemv_sequence_f16", 1, "a wait for earlier entries gave up: some workgroup was not "
+                             "resident (is another kernel occupying the compute units?)")
