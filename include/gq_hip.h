@@ -153,6 +153,21 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                          int64_t workspace_bytes, void *stream);
 
 /*
+ * gq_linear_kn_act_f16 for callers that cannot allocate device memory or pass a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The partial sums and arrival counters live in a device array
+ * inside the library (one copy per GPU, 16 KiB + GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES, held until the
+ * process ends); the call allocates and frees nothing.  Same arguments, results bit for bit those
+ * of gq_linear_kn_act_f16.  A problem whose gq_linear_kn_workspace_bytes() exceeds that size is
+ * rejected with GQ_ERR_UNSUPPORTED (decode batches of the 6B layer shapes fit up to 16 rows).
+ * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race.
+ */
+#define GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES (16 << 20)
+int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                                 int64_t k_in, int64_t group_size, int32_t activation, void *stream);
+
+/*
  * A sequence of decode GEMVs (a layer stack) as one call.  No counterpart in the reference, where
  * a model is a chain of LinearGQ.build calls (popxl_addons/layers/linear_gq.py:99-109) compiled
  * into one static device program; this entry point is the analogue for a chain of gq_gemv_f16

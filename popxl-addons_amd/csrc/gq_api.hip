@@ -192,6 +192,16 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                               workspace, (hipStream_t)stream);
 }
 
+int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                                 int64_t k_in, int64_t group_size, int32_t activation, void *stream) {
+  const int rc = check_linear_kn_args("gq_linear_kn_act_noalloc_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
+                                      k_in, group_size, activation);
+  if (rc <= 0) return rc;
+  return gq::launch_linear_kn_noalloc(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size,
+                                      (int)activation, (hipStream_t)stream);
+}
+
 static int gemv_sequence_common(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
                                 int32_t *status, void *workspace, int64_t spin_limit, void *stream) {
   if (count < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: negative count");

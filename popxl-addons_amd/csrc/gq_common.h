@@ -55,6 +55,9 @@ int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, i
 int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                      const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                      int64_t group_size, int act, void *workspace, hipStream_t stream);
+int launch_linear_kn_noalloc(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                             const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                             int64_t group_size, int act, hipStream_t stream);
 int64_t gemv_prepacked_bytes(int64_t n_out, int64_t k_in);
 int launch_gemv_prepack(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
                         int64_t k_in, hipStream_t stream);

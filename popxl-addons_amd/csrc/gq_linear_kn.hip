@@ -397,4 +397,44 @@ int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
   return check_launch("linear_kn_generic_kernel");
 }
 
+// ---------------------------------------------------------------------------------------
+// The same computation for callers that cannot hand over (or allocate) a workspace: the scratch
+// buffer is a device array of this library, one copy per GPU, held until the process ends.  Its
+// arrival counters are zero when the code object is loaded and every call leaves them zero; the
+// partial sums need no clearing (every word that is read was written by the same call).
+// Calls on one GPU share the array: calls that overlap (different streams) race.
+// ---------------------------------------------------------------------------------------
+constexpr int64_t kScratchBytes = (int64_t)kMaxStrips * 4 + GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+int launch_linear_kn_noalloc(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                             const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                             int64_t group_size, int act, hipStream_t stream) {
+  const int64_t need = linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
+  if (need > kScratchBytes)
+    return fail(GQ_ERR_UNSUPPORTED,
+                "gq_linear_kn_act_noalloc_f16: m_rows=%lld n_out=%lld k_in=%lld needs %lld bytes of scratch, the built-in "
+                "buffer holds %lld; use gq_linear_kn_act_f16 with a workspace",
+                (long long)m_rows, (long long)n_out, (long long)k_in, (long long)need, (long long)kScratchBytes);
+  void *ptr = nullptr;
+  if (need > 0) {
+    // the array's name is a host-side stand-in: its device address is looked up once per GPU, with
+    // that GPU current (every GPU has its own copy at its own address)
+    constexpr int kMaxDevices = 64;
+    static void *scratch_ptr[kMaxDevices] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
+    if (!scratch_ptr[dev]) {
+      void *p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !p) return fail(e == hipSuccess ? GQ_ERR_NO_DEVICE : (int)e, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+      scratch_ptr[dev] = p;
+    }
+    ptr = scratch_ptr[dev];
+  }
+  return launch_linear_kn(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, ptr, stream);
+}
+
 }  // namespace gq

@@ -41,6 +41,7 @@ EXPORTS = (
     "gq_linear_act_f16",
     "gq_linear_kn_workspace_bytes",
     "gq_linear_kn_act_f16",
+    "gq_linear_kn_act_noalloc_f16",
     "gq_gemv_sequence_f16",
     "gq_gemv_sequence_workspace_bytes",
     "gq_gemv_sequence_ws_f16",
@@ -98,6 +99,8 @@ def load():
     lib.gq_linear_kn_workspace_bytes.restype = i64
     lib.gq_linear_kn_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
     lib.gq_linear_kn_act_f16.restype = ctypes.c_int
+    lib.gq_linear_kn_act_noalloc_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p]
+    lib.gq_linear_kn_act_noalloc_f16.restype = ctypes.c_int
     lib.gq_gemv_sequence_f16.argtypes = [p, p, i64, p, p]
     lib.gq_gemv_sequence_f16.restype = ctypes.c_int
     lib.gq_gemv_sequence_workspace_bytes.argtypes = []

@@ -1,0 +1,73 @@
+"""gq_linear_kn_act_noalloc_f16: the fused matmul for weights grouped along the output features
+with its scratch buffer (partial sums, arrival counters) in a device array of the library, for
+callers that cannot allocate.  Checked through the C ABI against gq_linear_kn_act_f16 with a
+caller-provided workspace, bit for bit, on calls in a row that share the array -- the later ones
+smaller, so that they find the earlier ones' contents in it."""
+import numpy as np
+import pytest
+import torch
+
+from gq_testlib import activations, assert_bits_equal, to_dev
+from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(device, k_in, n_out, gs, m_rows, seed):
+    rng = np.random.default_rng(seed)
+    w = rng.normal(0, 0.02, (k_in, n_out)).astype(np.float16)
+    packed, scale, bias = group_quantize_compress_numpy(w, gs)
+    out_bias = rng.normal(0, 1, (n_out,)).astype(np.float16)
+    x = activations(m_rows, k_in, seed + 1)
+    return tuple(to_dev(a, device) for a in (x, packed, scale, bias, out_bias))
+
+
+def _with_workspace(hip, device, tensors, k_in, n_out, gs, m_rows, act):
+    x, packed, scale, bias, out_bias = tensors
+    need = hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, gs)
+    ws = torch.zeros(max(need, 16), dtype=torch.uint8, device=device)
+    y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    hip.call("gq_linear_kn_act_f16", x.data_ptr(), m_rows, packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+             out_bias.data_ptr(), y.data_ptr(), n_out, k_in, gs, act, ws.data_ptr(), ws.numel(),
+             torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return y.cpu().numpy(), need
+
+
+def _no_alloc(hip, device, tensors, k_in, n_out, gs, m_rows, act):
+    x, packed, scale, bias, out_bias = tensors
+    y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(device)
+    hip.call("gq_linear_kn_act_noalloc_f16", x.data_ptr(), m_rows, packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+             out_bias.data_ptr(), y.data_ptr(), n_out, k_in, gs, act, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated(device) == before
+    return y.cpu().numpy()
+
+
+def test_no_alloc_entry_point_matches_workspace_entry_point(hip, device):
+    # (k_in, n_out, group, m_rows, activation): a large problem first, then smaller ones that reuse
+    # the array with the first one's partial sums still in it, then a prefill batch (no scratch)
+    calls = [(4096, 16384, 64, 4, 0), (4096, 4096, 64, 2, 2), (1024, 2080, 32, 1, 1), (16384, 4096, 64, 16, 0),
+             (640, 544, 32, 3, 0), (512, 1024, 64, 40, 2)]
+    problems = [(_problem(device, k, n, gs, m, 100 + i), k, n, gs, m, act) for i, (k, n, gs, m, act) in enumerate(calls)]
+    want = [_with_workspace(hip, device, *p) for p in problems]
+    assert want[0][1] > 0 and want[-1][1] == 0
+    for _ in range(2):
+        for p, (y_want, _) in zip(problems, want):
+            assert_bits_equal(_no_alloc(hip, device, *p), y_want, str(p[1:]))
+
+
+def test_no_alloc_entry_point_rejects_oversized_problems(hip, device):
+    from popxl_addons._gq_hip import GQ_ERR_UNSUPPORTED, GQHipError
+
+    n_out, gs, m_rows = 153600, 64, 16  # 300 strips, two K slabs: 19.7 MB of partial sums
+    need = hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, 4096, gs)
+    assert need > (16 << 20) + 16384
+    tensors = _problem(device, 64, 64, gs, m_rows, 1)  # (never launched: the sizes are rejected first)
+    x, packed, scale, bias, out_bias = tensors
+    with pytest.raises(GQHipError) as e:
+        hip.call("gq_linear_kn_act_noalloc_f16", x.data_ptr(), m_rows, packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+                 0, x.data_ptr(), n_out, 4096, gs, 0, torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == GQ_ERR_UNSUPPORTED and "scratch" in str(e.value) and "workspace" in str(e.value)
