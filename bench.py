@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the 4-bit group-quantization path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decompress|gemv|gemm|stack|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decompress|compress|gemv|kn|gemm|stack|all]
 
 One "step" is one standalone int4 -> fp16 decompress of the 4096 x 16384 weight (benchmark
 configuration 2: group 64, ~N(0, 0.02) with 0.1 % outliers at +-8 sigma, packed by the
@@ -23,11 +23,35 @@ sys.path.insert(0, os.path.join(ROOT, "popxl-addons_amd"))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per decompress launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
-# each scaled by the same counter on a plain 128 MiB copy (read 36 880.7 KiB + written 131 295.8 KiB)
-DECOMPRESS_TRAFFIC_BYTES = int((36880.7 + 131295.8) * 1024)
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16, published
 GROUP = 64
+# HBM bytes per decompress launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: the summary
+# of those runs holds one machine-readable line with the figure and the commit it was taken at
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decompress_kernel_4096x16384.md")
+
+
+def measured_traffic():
+    """(bytes per launch, commit) from the committed profile summary, or (None, None)."""
+    import re
+
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)\s+at commit\s+([0-9a-f]{7,40})", text)
+    return (int(m.group(1)), m.group(2)) if m else (None, None)
+
+
+def hbm_roofline(kernel, nbytes, ms, **more):
+    gbs = nbytes / ms / 1e6
+    return dict({"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                 "frac": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes_per_launch": nbytes}, **more)
+
+
+def mfma_roofline(kernel, flops, ms, **more):
+    tf = flops / ms / 1e9
+    return dict({"kernel": kernel, "bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                 "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "algorithmic_flops_per_launch": flops}, **more)
 
 
 def log(*a):
@@ -101,13 +125,16 @@ def bench_decompress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384
     return {"ms": ms, "bytes": bytes_per_launch, "gbs": bytes_per_launch / ms / 1e6, "sets": sets}
 
 
-def bench_compress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384):
-    """Device-side packer on the configuration-2 weight: reads 2 B, writes 0.5 + 4/gs B per element."""
+def bench_compress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384, f32=False):
+    """Device-side packer on the configuration-2 weight: reads 2 B (4 B for float32 input), writes
+    0.5 + 4/gs B per element."""
     import torch
 
     sets = []
     for s in range(n_sets):
         w = make_weight(rows, cols, 100 + s, True, device)
+        if f32:
+            w = w.float()
         n_groups = cols // GROUP
         sets.append((w, torch.empty((rows, n_groups, GROUP // 4), dtype=torch.uint16, device=device),
                      torch.empty((rows, n_groups, 1), dtype=torch.float16, device=device),
@@ -117,28 +144,42 @@ def bench_compress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384):
 
     def step(i):
         w, p, s, b = sets[i % n_sets]
-        hip.call("gq_compress_f16", w.data_ptr(), p.data_ptr(), s.data_ptr(), b.data_ptr(), flag.data_ptr(), rows,
-                 cols // GROUP, GROUP, stream)
+        hip.call("gq_compress_f32" if f32 else "gq_compress_f16", w.data_ptr(), p.data_ptr(), s.data_ptr(), b.data_ptr(),
+                 flag.data_ptr(), rows, cols // GROUP, GROUP, stream)
 
     ms = time_launches(step, steps, warmup)
-    nbytes = rows * cols * (2.0 + 0.5 + 4.0 / GROUP)
-    return {"rows": rows, "cols": cols, "us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / ms / 1e6,
-            "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+    nbytes = rows * cols * ((4.0 if f32 else 2.0) + 0.5 + 4.0 / GROUP)
+    return {"rows": rows, "cols": cols, "input": "float32" if f32 else "float16", "us": ms * 1e3, "bytes": nbytes,
+            "gbs": nbytes / ms / 1e6, "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBS,
+            "roofline": hbm_roofline("compress_f32_kernel" if f32 else "compress_kernel", nbytes, ms)}
+
+
+def _blas_threads():
+    try:
+        from threadpoolctl import threadpool_info
+
+        return max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:  # noqa: BLE001 (a reporting aid only)
+        return None
+
+
+def _best_of(fn, repeats=3):
+    best, out = 1e30, None
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        out = fn()
+        best = min(best, time.perf_counter() - t0)
+    return best, out
 
 
 def cpu_baseline_decompress(sets, rows_sample=4096):
     """The numpy restatement of the reference's decompress (oracle/), timed on the host cores on one
     full 4096 x 16384 weight, best of 3.  numpy's elementwise passes run on one thread."""
-    import numpy as np
     from oracle import gq_oracle
 
     p, s, b, _ = sets[0]
     p, s, b = (a[:rows_sample].cpu().numpy() for a in (p, s, b))
-    best = 1e30
-    for _ in range(3):
-        t0 = time.perf_counter()
-        out = gq_oracle.np_decompress(p, s, b)
-        best = min(best, time.perf_counter() - t0)
+    best, out = _best_of(lambda: gq_oracle.np_decompress(p, s, b))
     n_bytes = p.nbytes + s.nbytes + b.nbytes + out.nbytes
     return {
         "value": n_bytes / best / 1e9,
@@ -150,35 +191,77 @@ def cpu_baseline_decompress(sets, rows_sample=4096):
     }, out
 
 
+def cpu_baseline_legs():
+    """The other CPU legs: configuration 1 decompress, and decompress -> float32 matmul (what the
+    reference's layer computes on the host, tests/integration/layers/test_linear_gq.py:18-30) for
+    configuration 3 (both shapes, batch 1) and configuration 4 (batch 128).  Same units as the
+    GPU rows they stand beside; seeded numpy inputs, the numpy packer."""
+    import numpy as np
+    from oracle import gq_oracle
+    from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy
+
+    rng = np.random.default_rng(1)
+    legs = []
+    w = rng.normal(0, 0.02, (1024, 1024)).astype(np.float16)
+    packed, scale, bias = group_quantize_compress_numpy(w, GROUP)
+    best, out = _best_of(lambda: gq_oracle.np_decompress(packed, scale, bias))
+    nbytes = packed.nbytes + scale.nbytes + bias.nbytes + out.nbytes
+    legs.append({"workload": "config 1: numpy decompress 1024x1024", "seconds": best, "value": nbytes / best / 1e9,
+                 "unit": "GB/s (read + written)", "cores": 1})
+    blas = _blas_threads()
+    for m_rows, n_out, k_in, name in ((1, 4096, 4096, "config 3"), (1, 16384, 4096, "config 3"), (128, 16384, 4096, "config 4")):
+        w = rng.normal(0, 0.02, (n_out, k_in)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, GROUP)
+        x = rng.normal(0, 1, (m_rows, k_in)).astype(np.float16)
+        best, _ = _best_of(lambda: gq_oracle.np_linear(x, gq_oracle.np_decompress(packed, scale, bias)), repeats=2)
+        w_bytes = n_out * k_in * (0.5 + 4.0 / GROUP)
+        legs.append({"workload": f"{name}: numpy decompress -> float32 matmul, m={m_rows} [{n_out}x{k_in}]", "seconds": best,
+                     "value": w_bytes / best / 1e9, "unit": "GB/s (packed weight bytes)",
+                     "tflops": 2.0 * m_rows * n_out * k_in / best / 1e12, "cores": f"decompress 1, BLAS {blas}"})
+    return legs
+
+
 # -------------------------------------------------------------------------------------- fused
 
 
-def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets):
-    """One fused dequant matmul shape; weights rotated over n_sets distinct copies."""
+def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets, kernel):
+    """One fused dequant matmul shape; weights rotated over n_sets distinct copies.  `entry` is
+    gq_gemv_f16 / gq_gemm_f16 (weight [n_out, k_in], groups along k_in) or gq_linear_kn_act_f16
+    (weight [k_in, n_out], groups along n_out: the default layout of LinearGQ)."""
     import torch
 
+    kn = entry == "gq_linear_kn_act_f16"
     sets = []
     for s in range(n_sets):
-        packed, scale, bias = pack_weight(make_weight(n_out, k_in, 200 + s, False, device))
-        sets.append((packed, scale, bias))
+        w = make_weight(k_in, n_out, 200 + s, False, device) if kn else make_weight(n_out, k_in, 200 + s, False, device)
+        sets.append(pack_weight(w))
     g = torch.Generator(device=device)
     g.manual_seed(7)
     x = torch.randn((m_rows, k_in), generator=g, device=device, dtype=torch.float32).to(torch.float16)
     y = torch.empty((m_rows, n_out), dtype=torch.float16, device=device)
     stream = stream_handle()
+    ws_bytes = hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, GROUP) if kn else 0
+    ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=device)
 
     def step(i):
         p, s, b = sets[i % n_sets]
-        hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP, stream)
+        if kn:
+            hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP,
+                     0, ws.data_ptr(), ws.numel(), stream)
+        else:
+            hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP, stream)
 
     ms = time_launches(step, steps, warmup)
     w_bytes = n_out * k_in * (0.5 + 4.0 / GROUP)
     flops = 2.0 * m_rows * n_out * k_in
-    return {
-        "m": m_rows, "n": n_out, "k": k_in, "us": ms * 1e3,
+    r = {
+        "m": m_rows, "n": n_out, "k": k_in, "layout": "[k_in, n_out]" if kn else "[n_out, k_in]", "us": ms * 1e3,
         "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
         "tflops": flops / ms / 1e9, "mfma_frac": flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
     }
+    # decode batches are bound by the packed weight bytes, prefill batches by the fp16 MFMA rate
+    r["roofline"] = hbm_roofline(kernel, w_bytes, ms) if m_rows <= 16 else mfma_roofline(kernel, flops, ms)
+    return r
 
 
 def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384):
@@ -277,6 +360,15 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
             seq.add(xs[k_in], p, s, b, ys[i % 6], None)
 
+    def free_streaming(seq):
+        # no dependencies, weights in the streaming layout, q k v fused: the ceiling of the kernel
+        for layer in range(n_layers):
+            w_qkv, w_o, w_up, w_down = prepacked[layer]
+            seq.add(xs[hidden], w_up, None, None, ys[4], None)
+            seq.add(xs[hidden], w_qkv, None, None, y_qkv, None)
+            seq.add(xs[ffn], w_down, None, None, ys[5], None)
+            seq.add(xs[hidden], w_o, None, None, ys[3], None)
+
     fused_qkv = [tuple(torch.cat([mats[layer * 6 + role][2 + part] for role in range(3)], dim=0).contiguous()
                        for part in range(3)) for layer in range(n_layers)]
     y_qkv = torch.empty((m_rows, 3 * hidden), dtype=torch.float16, device=device)
@@ -286,14 +378,33 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                        ("sequence_parallel_block_fused_qkv", parallel_fused_qkv),
                        ("sequence_parallel_block_fused_qkv_ffn_first", parallel_fused_qkv_ffn_first),
                        ("sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", parallel_fused_qkv_ffn_first_streaming),
-                       ("sequence_no_waits", free)):
+                       ("sequence_no_waits", free), ("sequence_no_waits_streaming_layout", free_streaming)):
         seq = hip.GemvSequence(device)
         fill(seq)
+        for y in ys + [y_qkv]:
+            y.fill_(float("nan"))
         ms = time_launches(lambda _: seq.run(), passes, warmup)
         torch.cuda.synchronize()
         results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                          "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
-                         "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0)}
+                         "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0),
+                         "roofline": hbm_roofline("gemv_stream_kernel", w_bytes, ms)}
+        # the timed passes computed something: what the buffers hold now (the last layer's outputs)
+        # equals single-call GEMVs on the same weights
+        worst = 0.0
+        last = (n_layers - 1) * 6
+        for role, y in ((3, ys[3]), (4, ys[4]), (5, ys[5])):
+            n_out, k_in, p, s, b = mats[last + role]
+            ref = torch.empty_like(y)
+            hip.call("gq_gemv_f16", xs[k_in].data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
+                     n_out, k_in, GROUP, stream_handle())
+            torch.cuda.synchronize()
+            worst = max(worst, ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item())
+        results[mode]["max_error_vs_single_call"] = worst
+        if not worst <= 2e-3 or results[mode]["status"] != 0:
+            raise SystemExit(f"bench.py: stack mode {mode} (m={m_rows}) is wrong: error {worst}, status {results[mode]['status']}")
+    results["per_launch_graph"]["roofline"] = hbm_roofline("gemv_mfma_kernel / gemv_stream_single_kernel (168 launches)", w_bytes,
+                                                           results["per_launch_graph"]["us_per_pass"] / 1e3)
     return results
 
 
@@ -302,7 +413,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", default="all", choices=["decompress", "gemv", "gemm", "stack", "all"])
+    ap.add_argument("--only", default="all", choices=["decompress", "compress", "gemv", "kn", "gemm", "stack", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB device copy (known traffic) for scaling profiler byte counters")
@@ -349,6 +460,10 @@ def main():
         same = np.array_equal(o.cpu().numpy().view(np.uint16), cpu_out.view(np.uint16))
         extra["gpu_equals_cpu_baseline_bits"] = bool(same)
         log(f"  {cpu['value']:.3f} GB/s on 1 core; GPU output bit-identical: {same}")
+        if args.only == "all":
+            cpu["legs"] = cpu_baseline_legs()
+            for leg in cpu["legs"]:
+                log(f"  cpu: {leg['workload']}: {leg['seconds']:.3f} s, {leg['value']:.3f} {leg['unit']}")
     if args.only == "all":
         # the same weight with the result transposed (dim=0 of the operator)
         outs_t = [torch.empty((16384, 4096), dtype=torch.float16, device=device) for _ in dec["sets"]]
@@ -360,29 +475,46 @@ def main():
 
         ms_t = time_launches(step_t, 100, 10)
         extra["decompress_transposed"] = {"rows": 4096, "cols": 16384, "us": ms_t * 1e3, "gbs": dec["bytes"] / ms_t / 1e6,
-                                          "hbm_frac": dec["bytes"] / ms_t / 1e6 / HBM_PEAK_GBS}
+                                          "hbm_frac": dec["bytes"] / ms_t / 1e6 / HBM_PEAK_GBS,
+                                          "roofline": hbm_roofline("decompress_transposed_tile_kernel", dec["bytes"], ms_t)}
         log(f"  transposed: {ms_t * 1e3:.1f} us, {dec['bytes'] / ms_t / 1e6:.0f} GB/s ({dec['bytes'] / ms_t / 1e6 / HBM_PEAK_GBS:.1%})")
         del outs_t
     del dec["sets"]
     torch.cuda.empty_cache()
 
-    if args.only == "all":
-        r = bench_compress(hip, device, 100, 10)
-        extra["compress"] = r
-        log(f"  compress 4096x16384: {r['us']:.1f} us, {r['gbs']:.0f} GB/s algorithmic ({r['hbm_frac']:.1%} of HBM peak)")
-        torch.cuda.empty_cache()
+    if args.only in ("compress", "all"):
+        for key, f32 in (("compress", False), ("compress_f32", True)):
+            r = bench_compress(hip, device, 100, 10, f32=f32)
+            extra[key] = r
+            log(f"  compress 4096x16384 from {r['input']}: {r['us']:.1f} us, {r['gbs']:.0f} GB/s algorithmic ({r['hbm_frac']:.1%} of HBM peak)")
+            torch.cuda.empty_cache()
     if args.only in ("gemv", "all"):
         extra["gemv"] = []
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
             for m in (1, 8):
-                r = bench_linear(hip, device, "gq_gemv_f16", m, n_out, k_in, 200, 20, n_sets=max(2, int(600e6 // (n_out * k_in * 0.5625)) + 1))
+                r = bench_linear(hip, device, "gq_gemv_f16", m, n_out, k_in, 200, 20,
+                                 n_sets=max(2, int(600e6 // (n_out * k_in * 0.5625)) + 1), kernel="gemv_mfma_kernel / gemv_stream_single_kernel")
                 extra["gemv"].append(r)
                 log(f"  gemv m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
+    if args.only in ("kn", "all"):
+        # the same shapes with the weight stored [k_in, n_out] and grouped along n_out: the default layout of LinearGQ
+        extra["linear_kn"] = []
+        for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
+            for m in (1, 8):
+                r = bench_linear(hip, device, "gq_linear_kn_act_f16", m, n_out, k_in, 200, 20,
+                                 n_sets=max(2, int(600e6 // (n_out * k_in * 0.5625)) + 1), kernel="gemv_kn_kernel")
+                extra["linear_kn"].append(r)
+                log(f"  kn-layout gemv m={m} [{k_in}->{n_out}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
+                torch.cuda.empty_cache()
+        r = bench_linear(hip, device, "gq_linear_kn_act_f16", 128, 16384, 4096, 30, 5, n_sets=2, kernel="gemm_kn_tile_kernel")
+        extra["linear_kn"].append(r)
+        log(f"  kn-layout gemm m=128 [4096->16384]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
+        torch.cuda.empty_cache()
     if args.only in ("gemm", "all"):
         extra["gemm"] = []
         for m in (128, 512, 2048):
-            r = bench_linear(hip, device, "gq_gemm_f16", m, 16384, 4096, 30, 5, n_sets=2)
+            r = bench_linear(hip, device, "gq_gemm_f16", m, 16384, 4096, 30, 5, n_sets=2, kernel="gemm_pipe2_kernel")
             extra["gemm"].append(r)
             log(f"  gemm m={m} [16384x4096]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
             torch.cuda.empty_cache()
@@ -392,12 +524,14 @@ def main():
             r = bench_stack(hip, device, m, passes=20, warmup=3)
             extra["stack"].append(r)
             for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block",
-                         "sequence_parallel_block_fused_qkv", "sequence_no_waits"):
+                         "sequence_parallel_block_fused_qkv", "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout",
+                         "sequence_no_waits", "sequence_no_waits_streaming_layout"):
                 log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
                     f"({r[mode]['hbm_frac']:.1%})")
             torch.cuda.empty_cache()
     extra["bench_wall_s"] = round(time.time() - t_begin, 1)
 
+    traffic, traffic_commit = measured_traffic()
     result = {
         "metric": "decompress GB/s & %HBM peak; fused dequant-GEMV/GEMM GB/s, TFLOP/s, %roofline",
         "value": round(dec["gbs"], 1),
@@ -422,7 +556,8 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(dec["gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": DECOMPRESS_TRAFFIC_BYTES,
+            "traffic": traffic,
+            "traffic_source": None if traffic is None else f"profiles/decompress_kernel_4096x16384.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {traffic_commit})",
             "kernel": "decompress_kernel",
             "algorithmic_bytes_per_launch": dec["bytes"],
         },

@@ -605,3 +605,75 @@ def test_gemv_sequences_with_own_workspaces_on_two_streams(hip, device, oracle):
                 w_dec = oracle.np_decompress(e[1].cpu().numpy(), e[2].cpu().numpy(), e[3].cpu().numpy())
                 assert_close(yy, oracle.np_linear(x_prev, w_dec, None if e[5] is None else e[5].cpu().numpy()), i)
             x_prev = yy
+
+
+@pytest.mark.parametrize("m_rows", [1, 4])
+def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows):
+    """The schedule the layer-stack benchmark times, on three full-size layers with real data flowing
+    through every declared wait: per layer the entries up (16384 x 4096, waits for the previous
+    layer), fused qkv (12288 x 4096), down (4096 x 16384, waits for up), o (4096 x 4096, waits for
+    qkv), every weight in the streaming layout.  up and qkv read the layer input, down reads up's
+    output, o reads 4096-wide rows out of qkv's output, and the next layer's input is o's output
+    (even layers) or down's (odd layers).  Every entry is checked against the oracle applied to the
+    inputs the device had; then the same sequence with the buffers of a role shared by all layers
+    (as the benchmark does: write-after-read hazards that only the declared waits resolve) must
+    end with the same bits."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    hidden, ffn, n_layers = 4096, 16384, 3
+    rng = np.random.default_rng(500 + m_rows)
+
+    def weight(n_out, k_in):
+        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        return oracle.np_decompress(packed, scale, bias), prepack_gemv(*(to_dev(a, device) for a in (packed, scale, bias)))
+
+    def out(n):
+        return torch.full((m_rows, n), float("nan"), dtype=torch.float16, device=device)
+
+    def v_rows(y_qkv):  # m_rows x 4096 contiguous values out of qkv's output, starting at its column 8192
+        return y_qkv.view(-1)[2 * hidden : 2 * hidden + m_rows * hidden].view(m_rows, hidden)
+
+    weights = [{name: weight(*shape) for name, shape in (("up", (ffn, hidden)), ("qkv", (3 * hidden, hidden)),
+                                                           ("down", (hidden, ffn)), ("o", (hidden, hidden)))} for _ in range(n_layers)]
+    h0 = to_dev(activations(m_rows, hidden, 9), device)
+
+    def build(shared_buffers):
+        seq, plan = GemvSequence(device), []
+        # shared: one up and one qkv buffer for all layers; o and down, which carry the layer input
+        # over to the next layer, alternate between two buffers (down of layer L + 1 does not wait
+        # for qkv of layer L + 1, which may still be reading down of layer L)
+        shared = [{"up": None, "qkv": None, "down": out(hidden), "o": out(hidden)} for _ in range(2)]
+        shared[0]["up"] = shared[1]["up"] = out(ffn)
+        shared[0]["qkv"] = shared[1]["qkv"] = out(3 * hidden)
+        h, last = h0, None
+        for layer in range(n_layers):
+            ys = shared[layer % 2] if shared_buffers else {"up": out(ffn), "qkv": out(3 * hidden), "down": out(hidden), "o": out(hidden)}
+            w = weights[layer]
+            up = seq.add(h, w["up"][1], None, None, ys["up"], wait_for=last)
+            qkv = seq.add(h, w["qkv"][1], None, None, ys["qkv"])
+            seq.add(ys["up"], w["down"][1], None, None, ys["down"], wait_for=up)
+            last = seq.add(v_rows(ys["qkv"]), w["o"][1], None, None, ys["o"], wait_for=qkv)
+            plan += [(h, w["up"][0], ys["up"]), (h, w["qkv"][0], ys["qkv"]), (ys["up"], w["down"][0], ys["down"]),
+                     (v_rows(ys["qkv"]), w["o"][0], ys["o"])]
+            h = ys["o"] if layer % 2 == 0 else ys["down"]
+        return seq, plan
+
+    seq, plan = build(shared_buffers=False)
+    assert [e[10] for e in seq.entries] == [0, 0, 1, 2, 4, 0, 5, 6, 8, 0, 9, 10]
+    for run in range(2):
+        for _, _, y in plan:
+            y.fill_(float("nan"))
+        seq.run()
+        seq.check()
+        for i, (x_in, w_dec, y) in enumerate(plan):
+            assert_close(y.cpu().numpy(), oracle.np_linear(x_in.cpu().numpy(), w_dec, None), (run, i))
+    final = [y.clone() for _, _, y in plan[-4:]]
+    shared_seq, shared_plan = build(shared_buffers=True)
+    for run in range(2):
+        for _, _, y in shared_plan[-4:]:
+            y.fill_(float("nan"))
+        shared_seq.run()
+        shared_seq.check()
+        for want, (_, _, y) in zip(final, shared_plan[-4:]):
+            assert torch.equal(want, y), run
