@@ -159,10 +159,11 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
  * inside the library (one copy per GPU, 16 KiB + GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES, held until the
  * process ends); the call allocates and frees nothing.  Same arguments, results bit for bit those
  * of gq_linear_kn_act_f16.  A problem whose gq_linear_kn_workspace_bytes() exceeds that size is
- * rejected with GQ_ERR_UNSUPPORTED (decode batches of the 6B layer shapes fit up to 16 rows).
+ * rejected with GQ_ERR_UNSUPPORTED (every problem of up to 8 rows fits; of the 6B layer shapes,
+ * 4096 and 16384 outputs fit up to 16 rows, the fused 12288-wide projection up to 8).
  * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race.
  */
-#define GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES (16 << 20)
+#define GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES (4 << 20)
 int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                                  int64_t k_in, int64_t group_size, int32_t activation, void *stream);

@@ -24,51 +24,59 @@ namespace {
 // ---------------------------------------------------------------------------------------
 // Decode kernel.  v_mfma_f32_16x16x32_f16: D[i][c] += sum_{kc, p} A[i][(kc, p)] * B[(kc, p)][c],
 // lane (i = lane % 16, kc = lane / 16) supplies A[i][(kc, 0..7)] and B[(kc, 0..7)][c = lane % 16].
-//   A: lane (i, kc) loads 16 bytes = 4 words = 32 outputs of input feature k0 + kc, at outputs
-//      n_strip + 32 i ..; word t of the lane is the A operand of MFMA t (dequantised, 8 fp16 in the
+//   A: lane (i, kc) loads 8 bytes = 2 words = 16 outputs of input feature k0 + kc, at outputs
+//      n_strip + 16 i ..; word t of the lane is the A operand of MFMA t (dequantised, 8 fp16 in the
 //      pair order (0,4,1,5,2,6,3,7) of their positions in the word).
 //   B: column c = (p', mm): position p' of a word, batch row mm of the pair the MFMA serves.
 //      B[(kc, p)][c] = x[mm][k0 + kc] if p == p' else 0 -- one non-zero half per lane.
-//   D_t[i][(p', mm)] = sum_kc W[k0 + kc][n_strip + 32 i + 8 t + order(p')] * x[mm][k0 + kc].
+//   D_t[i][(p', mm)] = sum_kc W[k0 + kc][n_strip + 16 i + 8 t + order(p')] * x[mm][k0 + kc].
 // One MFMA thus does 4 x 128 x 2 useful multiply-adds of its 8192: the matrix pipe has the room
-// (HBM delivers ~12 bytes per clock to a compute unit, 64 lanes x 16 bytes feed 4 MFMAs per batch
+// (HBM delivers ~12 bytes per clock to a compute unit; 64 lanes x 8 bytes feed 2 MFMAs per batch
 // pair), and the weights go from memory to the MFMA without a shuffle or an LDS round trip.
-// A wave covers a strip of 512 outputs (256 contiguous bytes per weight row, four rows per load
-// instruction); the 8 waves of a workgroup take every 8th block of 4 input features of the
-// workgroup's K slab.
+// A workgroup covers a strip of 256 outputs (128 contiguous bytes per weight row, four rows per
+// load instruction) and a slab of input features; its NW waves take every NW-th block of 4 input
+// features.  Narrow strips keep the cross-workgroup reduction small: one workgroup per compute
+// unit means (256 / strips) slabs, each leaving 2 KiB per batch-row pair for the strip's last
+// workgroup to add up.
 // ---------------------------------------------------------------------------------------
-constexpr int kStrip = 512;       // outputs per workgroup
+constexpr int kStrip = 256;       // outputs per workgroup
 constexpr int kMaxStrips = 4096;  // arrival counters at the start of the scratch buffer (16 KiB)
-constexpr int kKnWaves = 8;
-constexpr int kKnThreads = kKnWaves * 64;
 
-__device__ __forceinline__ float load_coherent(const float *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// device-coherent 16-byte accesses (sc1: written through to, and read from, the level of the memory
+// system that every compute unit sees): the partial sums of one workgroup are read by another
+// workgroup of the same launch
+__device__ __forceinline__ void store_coherent(float4_t *p, float4_t v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ void store_coherent(float *p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+template <int N>
+__device__ __forceinline__ void load_coherent(const float4_t *p, int64_t stride, float4_t (&v)[N]) {
+#pragma unroll
+  for (int j = 0; j < N; ++j) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[j]) : "v"(p + j * stride) : "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int j = 0; j < N; ++j) asm volatile("" : "+v"(v[j]));  // (uses of v stay below the wait)
 }
 
-// MP: batch-row pairs (m_rows <= 2 MP).  Scratch: one arrival counter per strip (zero before and
-// after every launch) and partial[split][m][n] fp32.
-template <int MP>
-__global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__restrict__ x, int m_rows,
-                                                             const char *__restrict__ packed,
-                                                             const half_t *__restrict__ scale,
-                                                             const half_t *__restrict__ bias,
-                                                             const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                             int n_out, int k_in, int gs_shift, int act, int slab,
-                                                             float *__restrict__ partial, unsigned *__restrict__ counters) {
-  __shared__ float4_t red[kKnWaves][4][64];
+// MP: batch-row pairs (m_rows <= 2 MP); NW: waves.  Scratch: one arrival counter per strip (zero
+// before and after every launch) and partial[split][strip][pair][t][lane] (a float4 each: the
+// accumulators as the lanes hold them).
+template <int MP, int NW>
+__global__ __launch_bounds__(NW * 64) void gemv_kn_kernel(const half_t *__restrict__ x, int m_rows,
+                                                          const char *__restrict__ packed, const half_t *__restrict__ scale,
+                                                          const half_t *__restrict__ bias, const half_t *__restrict__ out_bias,
+                                                          half_t *__restrict__ y, int n_out, int k_in, int gs_shift, int act,
+                                                          int slab, float4_t *__restrict__ partial,
+                                                          unsigned *__restrict__ counters) {
+  __shared__ float4_t red[NW][2][64];
   __shared__ unsigned arrived;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = lane & 15, kc = lane >> 4;
-  const int strip = blockIdx.x, split = blockIdx.y, n_splits = gridDim.y;
+  const int strip = blockIdx.x, n_strips = gridDim.x, split = blockIdx.y, n_splits = gridDim.y;
   const int n_groups = n_out >> gs_shift;
   const int64_t row_bytes = n_out >> 1;
-  // this lane's 32 outputs; lanes past n_out re-read the last 16 bytes of the row (results dropped)
-  const int n_lane = strip * kStrip + 32 * i;
-  const int n_load = min(n_lane, n_out - 32);
+  // this lane's 16 outputs; lanes past n_out re-read the last 8 bytes of the row (results dropped)
+  const int n_lane = strip * kStrip + 16 * i;
+  const int n_load = min(n_lane, n_out - 16);
   const int g_lane = n_load >> gs_shift;
   const int k_begin = split * slab, k_end = min(k_in, k_begin + slab);
 
@@ -78,24 +86,24 @@ __global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__res
 #pragma unroll
   for (int r = 0; r < 4; ++r) mask[r] = (p_sel >> 1) == r ? ((p_sel & 1) ? 0xFFFF0000u : 0x0000FFFFu) : 0u;
 
-  float4_t acc[MP][4];
+  float4_t acc[MP][2];
 #pragma unroll
   for (int mp = 0; mp < MP; ++mp)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[mp][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < 2; ++t) acc[mp][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   // U blocks of 4 input features per iteration, every load of them issued before the first use:
-  // a wave keeps U KiB of weights in flight
-  constexpr int U = MP <= 2 ? 4 : 2;
-  for (int kb = k_begin + 4 * wave; kb < k_end; kb += 4 * kKnWaves * U) {
-    uint4_t wq[U];
+  // a wave keeps U x 512 bytes of weights in flight
+  constexpr int U = MP <= 2 ? 8 : (MP <= 4 ? 4 : 2);
+  for (int kb = k_begin + 4 * wave; kb < k_end; kb += 4 * NW * U) {
+    uint2_t wq[U];
     uint32_t sv[U], bv[U], xv[U][MP];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = kb + 4 * kKnWaves * u + kc;
+      const int k = kb + 4 * NW * u + kc;
       const bool live = k < k_end;
       const int kk = live ? k : k_end - 1;  // (past the slab: any valid row, multiplied by x = 0)
-      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t *>(packed + kk * row_bytes + (n_load >> 1)));
+      wq[u] = __builtin_nontemporal_load(reinterpret_cast<const uint2_t *>(packed + kk * row_bytes + (n_load >> 1)));
       sv[u] = __builtin_bit_cast(uint16_t, scale[(int64_t)kk * n_groups + g_lane]);
       bv[u] = __builtin_bit_cast(uint16_t, bias[(int64_t)kk * n_groups + g_lane]);
 #pragma unroll
@@ -107,9 +115,9 @@ __global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__res
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const half2_t s2 = as_half2(sv[u] | (sv[u] << 16)), b2 = as_half2(bv[u] | (bv[u] << 16));
-      half8_t a[4];
+      half8_t a[2];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) a[t] = dequant_word(wq[u][t], s2, b2);
+      for (int t = 0; t < 2; ++t) a[t] = dequant_word(wq[u][t], s2, b2);
 #pragma unroll
       for (int mp = 0; mp < MP; ++mp) {
         const uint32_t xx = xv[u][mp] | (xv[u][mp] << 16);
@@ -118,42 +126,43 @@ __global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__res
         for (int r = 0; r < 4; ++r) bq[r] = xx & mask[r];
         const half8_t b = __builtin_bit_cast(half8_t, bq);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[mp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t], b, acc[mp][t], 0, 0, 0);
+        for (int t = 0; t < 2; ++t) acc[mp][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t], b, acc[mp][t], 0, 0, 0);
       }
     }
   }
 
   // lane (c, rg) of accumulator (mp, t) holds, in element e, row i = 4 rg + e: the output
-  // n = strip + 32 i + 8 t + order(p'), batch row m = 2 mp + mm.  The waves' sums meet in LDS, one
-  // batch-row pair at a time.
+  // n = strip + 16 i + 8 t + order(p'), batch row m = 2 mp + mm.  The waves' sums meet in LDS, one
+  // batch-row pair at a time; threads 0..127 then own one float4 (t, lane) each.
   const bool direct = n_splits == 1;
+  const int ot = (threadIdx.x >> 6) & 1, ol = threadIdx.x & 63;
+  auto finish = [&](int mp, float4_t sum) {  // sum + out_bias -> activation -> y
+    const int cc = ol & 15, rg = ol >> 4;
+    const int m = 2 * mp + (cc & 1);
+    if (m >= m_rows) return;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // position p' = cc / 2 of a word holds its element p' / 2 + 4 (p' % 2)
+      const int n = strip * kStrip + 16 * (4 * rg + e) + 8 * ot + (cc >> 2) + 4 * ((cc >> 1) & 1);
+      if (n >= n_out) continue;
+      float v = sum[e];
+      if (out_bias) v += (float)out_bias[n];
+      y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
+    }
+  };
+  float4_t *mine = partial + (((int64_t)split * n_strips + strip) * MP) * 128 + threadIdx.x;
 #pragma unroll
   for (int mp = 0; mp < MP; ++mp) {
     if (mp > 0) __syncthreads();
 #pragma unroll
-    for (int t = 0; t < 4; ++t) red[wave][t][lane] = acc[mp][t];
+    for (int t = 0; t < 2; ++t) red[wave][t][lane] = acc[mp][t];
     __syncthreads();
-    if (threadIdx.x < 256) {
-      const int l = threadIdx.x & 63, t = threadIdx.x >> 6;
-      float4_t sum = red[0][t][l];
+    if (threadIdx.x < 128) {
+      float4_t sum = red[0][ot][ol];
 #pragma unroll
-      for (int w = 1; w < kKnWaves; ++w) sum += red[w][t][l];
-      const int cc = l & 15, rg = l >> 4;
-      const int m = 2 * mp + (cc & 1);
-      if (m < m_rows) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int n = strip * kStrip + 32 * (4 * rg + e) + 8 * t + (cc >> 2) + 4 * ((cc >> 1) & 1);  // position p' = cc / 2 holds element p' / 2 + 4 (p' % 2)
-          if (n >= n_out) continue;
-          if (direct) {
-            float v = sum[e];
-            if (out_bias) v += (float)out_bias[n];
-            y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
-          } else {
-            store_coherent(partial + ((int64_t)split * m_rows + m) * n_out + n, sum[e]);
-          }
-        }
-      }
+      for (int w = 1; w < NW; ++w) sum += red[w][ot][ol];
+      if (direct) finish(mp, sum);
+      else store_coherent(mine + mp * 128, sum);
     }
   }
   if (direct) return;
@@ -167,15 +176,27 @@ __global__ __launch_bounds__(kKnThreads) void gemv_kn_kernel(const half_t *__res
       __hip_atomic_store(counters + strip, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
-  if (arrived != (unsigned)n_splits - 1) return;
-  // last workgroup of the strip: add the splits in order (the same result whoever arrives last)
-  const int n_strip = min(kStrip, n_out - strip * kStrip);
-  for (int o = threadIdx.x; o < m_rows * n_strip; o += kKnThreads) {
-    const int m = o / n_strip, n = strip * kStrip + o % n_strip;
-    float v = 0.f;
-    for (int s = 0; s < n_splits; ++s) v += load_coherent(partial + ((int64_t)s * m_rows + m) * n_out + n);
-    if (out_bias) v += (float)out_bias[n];
-    y[(int64_t)m * n_out + n] = (half_t)apply_activation(v, act);
+  if (arrived != (unsigned)n_splits - 1 || threadIdx.x >= 128) return;
+  // last workgroup of the strip: add the slabs in order (the same result whoever arrives last),
+  // eight loads in flight at a time
+  const int64_t stride = (int64_t)n_strips * MP * 128;  // float4 between consecutive slabs
+  const float4_t *first = partial + ((int64_t)strip * MP) * 128 + threadIdx.x;
+#pragma unroll
+  for (int mp = 0; mp < MP; ++mp) {
+    float4_t sum = {0.f, 0.f, 0.f, 0.f};
+    int s = 0;
+    for (; s + 8 <= n_splits; s += 8) {
+      float4_t v[8];
+      load_coherent<8>(first + mp * 128 + s * stride, stride, v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += v[j];
+    }
+    for (; s < n_splits; ++s) {
+      float4_t v[1];
+      load_coherent<1>(first + mp * 128 + s * stride, stride, v);
+      sum += v[0];
+    }
+    finish(mp, sum);
   }
 }
 
@@ -317,17 +338,22 @@ __global__ __launch_bounds__(256) void gemm_kn_tile_kernel(const half_t *__restr
     }
 }
 
-// K slabs of the decode kernel: enough workgroups to fill the device twice over, slabs a multiple
-// of the 32 input features that the 8 waves take per round
-int kn_splits(int64_t n_out, int64_t k_in, int64_t *slab_out) {
+// waves of the decode kernel for a batch (the 16 accumulator registers per batch-row pair of the
+// largest batches leave room for 8 waves' worth of registers only)
+int kn_waves(int64_t m_rows) { return m_rows <= 8 ? 16 : 8; }
+int kn_pairs(int64_t m_rows) { return m_rows <= 2 ? 1 : (m_rows <= 4 ? 2 : (m_rows <= 8 ? 4 : 8)); }
+
+// K slabs of the decode kernel: one workgroup per compute unit (256), slabs a multiple of the input
+// features that the waves take per round, at least two rounds per wave
+int kn_splits(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t *slab_out) {
+  const int64_t round = 4 * kn_waves(m_rows);
   const int64_t strips = (n_out + kStrip - 1) / kStrip;
-  int64_t splits = (512 + strips - 1) / strips;  // two workgroups per compute unit
-  const int64_t max_splits = (k_in + 127) / 128;  // at least four rounds per wave
+  int64_t splits = (256 + strips - 1) / strips;
+  const int64_t max_splits = (k_in + 2 * round - 1) / (2 * round);
   if (splits > max_splits) splits = max_splits;
-  if (splits > 64) splits = 64;
   if (splits < 1) splits = 1;
   int64_t slab = (k_in + splits - 1) / splits;
-  slab = (slab + 31) / 32 * 32;
+  slab = (slab + round - 1) / round * round;
   splits = (k_in + slab - 1) / slab;
   *slab_out = slab;
   return (int)splits;
@@ -342,16 +368,17 @@ bool kn_fast_shape(const uint16_t *x, const uint16_t *packed, int64_t n_out, int
 }  // namespace
 
 // Scratch bytes the decode kernel needs for this problem (0: none): the arrival counters (a fixed
-// 16 KiB at the start, so that calls of any shape find them at the same place), then fp32 partial
-// sums per K slab.
+// 16 KiB at the start, so that calls of any shape find them at the same place), then 2 KiB of
+// fp32 partial sums per (K slab, strip, batch-row pair).
 int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
   if (m_rows < 1 || m_rows > 16 || k_in < 1) return 0;
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   if (!pow2 || group_size < 32 || n_out % 32 != 0 || n_out < 32 || n_out > (int64_t)kMaxStrips * kStrip) return 0;
   int64_t slab = 0;
-  const int splits = kn_splits(n_out, k_in, &slab);
+  const int splits = kn_splits(m_rows, n_out, k_in, &slab);
   if (splits == 1) return 0;
-  return (int64_t)kMaxStrips * 4 + splits * m_rows * n_out * 4;
+  const int64_t strips = (n_out + kStrip - 1) / kStrip;
+  return (int64_t)kMaxStrips * 4 + splits * strips * kn_pairs(m_rows) * 2048;
 }
 
 // `workspace`: linear_kn_workspace_bytes() bytes of device memory whose first 16 KiB (the counters)
@@ -366,18 +393,19 @@ int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
   const int gs_shift = fast ? __builtin_ctzll((unsigned long long)group_size) : 0;
   if (fast && m_rows <= 16) {
     int64_t slab = 0;
-    const int splits = kn_splits(n_out, k_in, &slab);
+    const int splits = kn_splits(m_rows, n_out, k_in, &slab);
     const int64_t strips = (n_out + kStrip - 1) / kStrip;
     unsigned *counters = static_cast<unsigned *>(workspace);
-    float *partial = reinterpret_cast<float *>(counters + kMaxStrips);
-    const dim3 grid((unsigned)strips, (unsigned)splits), block(kKnThreads);
-#define GQ_KN(MP)                                                                                                    \
-  gemv_kn_kernel<MP><<<grid, block, 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, oh, yh, \
-                                                 (int)n_out, (int)k_in, gs_shift, act, (int)slab, partial, counters)
-    if (m_rows <= 2) GQ_KN(1);
-    else if (m_rows <= 4) GQ_KN(2);
-    else if (m_rows <= 8) GQ_KN(4);
-    else GQ_KN(8);
+    float4_t *partial = reinterpret_cast<float4_t *>(counters + kMaxStrips);
+    const dim3 grid((unsigned)strips, (unsigned)splits);
+#define GQ_KN(MP, NW)                                                                                                       \
+  gemv_kn_kernel<MP, NW><<<grid, dim3(NW * 64), 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, \
+                                                             oh, yh, (int)n_out, (int)k_in, gs_shift, act, (int)slab, partial, \
+                                                             counters)
+    if (m_rows <= 2) GQ_KN(1, 16);
+    else if (m_rows <= 4) GQ_KN(2, 16);
+    else if (m_rows <= 8) GQ_KN(4, 16);
+    else GQ_KN(8, 8);
 #undef GQ_KN
     return check_launch("gemv_kn_kernel");
   }

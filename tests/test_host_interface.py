@@ -61,7 +61,7 @@ def test_abi_version_and_error_text_without_gpu():
     assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "activation" in str(e.value)
     need = lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 64)
     assert need > 16384 and need <= 16384 + 64 * 16384 * 4 and need == lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 32)
-    assert lib.gq_linear_kn_workspace_bytes(4, 16384, 4096, 64) == 16384 + (need - 16384) * 4
+    assert lib.gq_linear_kn_workspace_bytes(4, 16384, 4096, 64) == 16384 + (need - 16384) * 2  # two batch-row pairs
     assert lib.gq_linear_kn_workspace_bytes(1, 128, 64, 64) == 0  # one K slab: no scratch
     assert lib.gq_linear_kn_workspace_bytes(17, 16384, 4096, 64) == 0  # prefill batches need none
     assert lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 20) == 0  # generic kernel

@@ -62,9 +62,9 @@ def test_no_alloc_entry_point_matches_workspace_entry_point(hip, device):
 def test_no_alloc_entry_point_rejects_oversized_problems(hip, device):
     from popxl_addons._gq_hip import GQ_ERR_UNSUPPORTED, GQHipError
 
-    n_out, gs, m_rows = 153600, 64, 16  # 300 strips, two K slabs: 19.7 MB of partial sums
+    n_out, gs, m_rows = 12288, 64, 16  # 48 strips x 6 K slabs x 8 batch-row pairs x 2 KiB = 4.5 MiB of partial sums
     need = hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, 4096, gs)
-    assert need > (16 << 20) + 16384
+    assert need > (4 << 20) + 16384
     tensors = _problem(device, 64, 64, gs, m_rows, 1)  # (never launched: the sizes are rejected first)
     x, packed, scale, bias, out_bias = tensors
     with pytest.raises(GQHipError) as e:
