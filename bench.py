@@ -308,6 +308,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     #                      these shapes is built that way): order q k v up o down; q waits for the
     #                      previous layer, o for v (up streams meanwhile), down for up
     #   ... fused qkv       the parallel block with q, k, v as one 12288 x 4096 entry: 112 entries per pass
+    #   decoder data flow  the fused-qkv, ffn-first schedule with every entry reading what its predecessor
+    #                      wrote (results travel through the kernel's tagged exchange: no reported completion)
     #   no waits           no dependencies: the streaming rate of the kernel alone, not a decoder
     def sequential(seq):
         for i, (n_out, k_in, p, s, b) in enumerate(mats):
@@ -374,14 +376,39 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     y_qkv = torch.empty((m_rows, 3 * hidden), dtype=torch.float16, device=device)
     prepacked = [(hip.prepack_gemv(*fused_qkv[layer]),) + tuple(hip.prepack_gemv(*mats[layer * 6 + role][2:]) for role in (3, 4, 5))
                  for layer in range(n_layers)]
+    # the decoder schedule with DATA flowing through every wait: up and qkv read the layer input h,
+    # down reads up's output, o reads 4096-wide rows out of qkv's output, and o's output is the next
+    # layer's h.  (h starts small: without normalisation layers every layer multiplies it by 1.6.)
+    g.manual_seed(11)
+    h0 = (torch.randn((m_rows, hidden), generator=g, device=device, dtype=torch.float32) * 1e-3).to(torch.float16)
+    y_o2 = [torch.empty((m_rows, hidden), dtype=torch.float16, device=device) for _ in range(2)]
+
+    def v_rows(t):
+        return t.view(-1)[2 * hidden : 2 * hidden + m_rows * hidden].view(m_rows, hidden)
+
+    def data_flow(seq, streaming=True):
+        h, last = h0, None
+        for layer in range(n_layers):
+            if streaming:
+                w_qkv, w_o, w_up, w_down = ((w, None, None) for w in prepacked[layer])
+            else:
+                w_qkv, w_o, w_up, w_down = fused_qkv[layer], mats[layer * 6 + 3][2:], mats[layer * 6 + 4][2:], mats[layer * 6 + 5][2:]
+            b_ = seq.add(h, *w_up, ys[4], None, wait_for=last)
+            a = seq.add(h, *w_qkv, y_qkv, None)
+            seq.add(ys[4], *w_down, ys[5], None, wait_for=b_)
+            last = seq.add(v_rows(y_qkv), *w_o, y_o2[layer % 2], None, wait_for=a)
+            h = y_o2[layer % 2]
+
     for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
                        ("sequence_parallel_block_fused_qkv", parallel_fused_qkv),
                        ("sequence_parallel_block_fused_qkv_ffn_first", parallel_fused_qkv_ffn_first),
                        ("sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", parallel_fused_qkv_ffn_first_streaming),
+                       ("sequence_decoder_data_flow", lambda seq: data_flow(seq, streaming=False)),
+                       ("sequence_decoder_data_flow_streaming_layout", data_flow),
                        ("sequence_no_waits", free), ("sequence_no_waits_streaming_layout", free_streaming)):
         seq = hip.GemvSequence(device)
         fill(seq)
-        for y in ys + [y_qkv]:
+        for y in ys + [y_qkv] + y_o2:
             y.fill_(float("nan"))
         ms = time_launches(lambda _: seq.run(), passes, warmup)
         torch.cuda.synchronize()
@@ -390,13 +417,18 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                          "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0),
                          "roofline": hbm_roofline("gemv_stream_kernel", w_bytes, ms)}
         # the timed passes computed something: what the buffers hold now (the last layer's outputs)
-        # equals single-call GEMVs on the same weights
+        # equals single-call GEMVs on the same weights and the inputs the device had
         worst = 0.0
         last = (n_layers - 1) * 6
-        for role, y in ((3, ys[3]), (4, ys[4]), (5, ys[5])):
+        if "data_flow" in mode:
+            h_last = y_o2[(n_layers - 2) % 2]
+            checks = ((3, v_rows(y_qkv), y_o2[(n_layers - 1) % 2]), (4, h_last, ys[4]), (5, ys[4], ys[5]))
+        else:
+            checks = tuple((role, xs[mats[last + role][1]], ys[role]) for role in (3, 4, 5))
+        for role, x_in, y in checks:
             n_out, k_in, p, s, b = mats[last + role]
             ref = torch.empty_like(y)
-            hip.call("gq_gemv_f16", xs[k_in].data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
+            hip.call("gq_gemv_f16", x_in.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
                      n_out, k_in, GROUP, stream_handle())
             torch.cuda.synchronize()
             worst = max(worst, ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item())
@@ -525,6 +557,7 @@ def main():
             extra["stack"].append(r)
             for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block",
                          "sequence_parallel_block_fused_qkv", "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout",
+                         "sequence_decoder_data_flow", "sequence_decoder_data_flow_streaming_layout",
                          "sequence_no_waits", "sequence_no_waits_streaming_layout"):
                 log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
                     f"({r[mode]['hbm_frac']:.1%})")

@@ -59,13 +59,33 @@ constexpr int kStageBytes = 4096;       // x stage of a wave: 1 KiB per (chunk, 
 // more hop for a wait that is exposed; measured: one watcher beats eight, and a watcher workgroup
 // without rows of its own loses more to the uneven split of the row blocks than it gains).
 constexpr int kMaxGroups = 256;  // (the watcher keeps a copy of every progress word in LDS)
+constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
 constexpr int kProgressStride = 32;  // words
 // layout of the block: [kMaxGroups] progress lines, the watcher's announcement, the count of
 // workgroups that have left the kernel (a line each); all zero between launches
 constexpr int kAnnouncedWord = kMaxGroups * kProgressStride;
 constexpr int kExitedWord = kAnnouncedWord + kProgressStride;
-constexpr int kSequenceWords = kExitedWord + kProgressStride;
+constexpr int kEpochWord = kExitedWord + kProgressStride;
+// The exchange: results that a later entry of the same launch reads as its x are also written here
+// as 32-bit words (tag << 16 | fp16 value), the tag being the launch's epoch (1..65535, kept in the
+// block, advanced by the last workgroup to leave).  A consumer loads the words and knows from the
+// tags alone that every value has arrived: no wait for the producers' stores to complete, no
+// progress report, no reload of x after a flag -- three memory round trips less per dependency.
+// Stale words carry older tags; when the epoch wraps, the last workgroup out clears the exchange.
+constexpr int kExchangeWord = (kEpochWord + kProgressStride + 63) / 64 * 64;  // 256-byte aligned
+constexpr int kExchangeWords = (16 << 20) / 4;
+constexpr int kSequenceWords = kExchangeWord + kExchangeWords;
 __device__ __attribute__((aligned(256))) unsigned int g_sequence_words[kSequenceWords];
+
+// What the host works out for a launch (a kernel argument): which entries read results of the
+// launch through the exchange, and which have to wait for reported completion.
+struct SequencePlan {
+  int32_t ex_word[kMaxEntries];  // producer: where the entry's tagged results start in the exchange (-1: none)
+  int32_t x_word[kMaxEntries];   // consumer: where its x starts in the exchange (-1: x is read from memory)
+  int16_t x_src[kMaxEntries];    // consumer: the entry (of this launch) that produces its x (-1: none)
+  int16_t need[kMaxEntries];     // entries of this launch that must be reported complete before this one starts
+  int32_t uses_exchange;
+};
 
 struct Entry {  // = gq_gemv_desc
   const half_t *x;
@@ -101,7 +121,6 @@ struct CachedEntry {
   char act;            // GQ_ACT_* epilogue
 };
 static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
-constexpr int kMaxEntries = 128;  // per launch (8 KiB of LDS)
 
 // cache policy of a direct-to-LDS load: sc1 = device (agent) scope, the policy the compiler gives an
 // agent-scope atomic load; it pairs with the agent-scope stores of y and of the progress words
@@ -113,9 +132,11 @@ struct Control {
   unsigned deposited[2];  // mailbox deposits so far, passes of even and of odd number (8 per pass)
   unsigned consumed;      // passes whose mailboxes the reducer has read
   unsigned ready;         // entries known to be complete on the whole device
-  unsigned failed;        // the poller gave up
+  unsigned failed;        // a poller gave up
   unsigned published;     // entries this workgroup has reported complete (progress word written)
   unsigned targets[4];    // bit w - 1 set: some entry waits for the first w entries (kMaxEntries bits)
+  unsigned tag;           // this launch's epoch << 16
+  unsigned stored;        // entries whose results this workgroup's reducer has stored (stores issued)
 };
 static_assert(sizeof(Control) <= 64, "control block");
 
@@ -174,9 +195,9 @@ __device__ __forceinline__ half8_t raw_codes(uint32_t w, uint32_t mask_lo, uint3
 // publishes, and x is read with device-coherent loads.
 // SINGLE: the sequence is the one entry `single`, passed by value (no descriptor in memory).
 template <int MC, int NS, bool SINGLE>
-__device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries, int first_entry,
-                                                 int *__restrict__ status, unsigned *__restrict__ words,
-                                                 unsigned spin_limit, const Entry single) {
+__device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entries, int n_entries,
+                                                 int *__restrict__ status, unsigned *words, unsigned spin_limit,
+                                                 const SequencePlan *plan, const Entry single) {
   static_assert(MC == 2 || MC == 4, "batch capacity");
   constexpr int PR = pass_rows(MC);
   extern __shared__ __attribute__((aligned(64))) char lds[];
@@ -188,6 +209,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   const int r = lane & 15, kc = lane >> 4;
   const int G = gridDim.x, b = blockIdx.x;
   unsigned *const g_progress = words, *const g_announced = words + kAnnouncedWord, *const g_exited = words + kExitedWord;
+  unsigned *const g_epoch = words + kEpochWord, *const exchange = words + kExchangeWord;
   CachedEntry *cache = reinterpret_cast<CachedEntry *>(lds + kWaves * kWaveBytes);
   float *mail = reinterpret_cast<float *>(lds + kWaves * kWaveBytes + kMaxEntries * 64);
   Control *ctl = reinterpret_cast<Control *>(mail + 2 * kWaves * kMailFloats);  // two sets of mailboxes
@@ -209,7 +231,7 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     c.n_out = e.n_out;
     c.k_in = e.k_in;
     c.m_rows = (short)e.m_rows;
-    c.wait = (short)max(0, e.wait_entries - first_entry);  // earlier launches are complete
+    c.wait = SINGLE ? (short)0 : plan->need[i];  // (entries of earlier launches are complete)
     const int rb = (e.n_out + 15) >> 4;
     c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
     c.publish = 0;
@@ -217,7 +239,14 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
     cache[i] = c;
   }
   if (tid < kMaxGroups) seen[tid] = 0u;
-  if (tid == 0) *ctl = Control{{0u, 0u}, 0u, 0u, 0u, 0u, {0u, 0u, 0u, 0u}};
+  if (tid == 0) {
+    unsigned tag = 0;
+    if (!SINGLE && plan->uses_exchange) {
+      tag = __hip_atomic_load(g_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tag == 0) tag = 1;  // a fresh block
+    }
+    *ctl = Control{{0u, 0u}, 0u, 0u, 0u, 0u, {0u, 0u, 0u, 0u}, tag << 16, 0u};
+  }
   __syncthreads();
   // completion is reported only where an entry waits for it (a report costs the reducer a round
   // trip to memory)
@@ -323,6 +352,10 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       half_t *y = cache[d].y;
       const half_t *out_bias = cache[d].out_bias;
       const int act = uni(cache[d].act);
+      // a later entry of this launch reads these results as its x: they also go to the exchange, tagged
+      const int ex_word = SINGLE ? -1 : plan->ex_word[d];
+      unsigned *const ex = ex_word >= 0 ? exchange + ex_word : nullptr;
+      const unsigned tag = ex ? (unsigned)uni((int)lds_load(&ctl->tag)) : 0u;
       for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
         const int nj = min(PR, nrb - pass * PR);
         while (lds_load(&ctl->deposited[q & 1]) < ((q >> 1) + 1) * kWaves) __builtin_amdgcn_s_sleep(1);
@@ -340,12 +373,17 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
             // device-scope store: written through to where every compute unit reads it
             __hip_atomic_store(reinterpret_cast<unsigned short *>(y) + (int64_t)m * n_out + n,
                                __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (ex)
+              __hip_atomic_store(ex + (int64_t)m * n_out + n, tag | __builtin_bit_cast(unsigned short, hv), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
           }
         }
         // the mailboxes have been read (the sums above depend on them): free them
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) __hip_atomic_store(&ctl->consumed, q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
+      // (consumers in this workgroup start to look for the results on the whole device from here)
+      if (ex && lane == 0) __hip_atomic_store(&ctl->stored, (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (uni(cache[d].publish)) {
         wait_vm<0>();  // every lane's stores of this and of all earlier entries are complete ...
         if (lane == 0) {  // ... then publish
@@ -354,18 +392,34 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
         }
       }
     }
-    // a sequence without dependencies has not touched the progress words
+    // a sequence without dependencies has touched neither the progress words nor the exchange
     const unsigned any_target = ctl->targets[0] | ctl->targets[1] | ctl->targets[2] | ctl->targets[3];
-    if (uni((int)any_target) == 0) return;
-    // the last workgroup out clears the progress words: by then every poller has seen all it needs
+    const bool uses_exchange = !SINGLE && plan->uses_exchange;
+    if (uni((int)any_target) == 0 && !uses_exchange) return;
+    // the last workgroup out clears the progress words and advances the epoch: by then every
+    // poller has seen all it needs and nobody reads the exchange any more (a workgroup's compute
+    // waves have finished before its reducer gets here)
     wait_vm<0>();  // this workgroup's last progress word is in memory before it counts itself out
     unsigned last = 0;
     if (lane == 0) last = atomicAdd(g_exited, 1u) == (unsigned)G - 1;
     if (uni((int)last)) {
       wait_vm<0>();
-      for (int i = lane; i < G; i += 64)
-        __hip_atomic_store(&g_progress[i * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (lane == 0) __hip_atomic_store(g_announced, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (uni((int)any_target)) {
+        for (int i = lane; i < G; i += 64)
+          __hip_atomic_store(&g_progress[i * kProgressStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(g_announced, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if (uses_exchange) {
+        unsigned epoch = (unsigned)uni((int)lds_load(&ctl->tag)) >> 16;
+        if (epoch == 0xFFFFu) {
+          // the tags are about to repeat: no word of an earlier launch may survive
+          for (int i = lane; i < kExchangeWords / 4; i += 64)
+            __builtin_nontemporal_store(uint4_t{0u, 0u, 0u, 0u}, reinterpret_cast<uint4_t *>(exchange) + i);
+          wait_vm<0>();
+          epoch = 0;
+        }
+        if (lane == 0) __hip_atomic_store(g_epoch, epoch + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       if (lane == 0) __hip_atomic_store(g_exited, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     return;
@@ -496,6 +550,60 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
   const half_t *st_x = nullptr;  // the stage holds this wave's chunk of EVERY phase of (st_x, st_k, st_m)
   int st_k = 0, st_m = 0;
   unsigned known_ready = 0;  // entries this wave has seen complete on the whole device
+  int x_from = -1;           // the entry of this launch that produced the x in the registers / the stage (-1: memory)
+
+  // Rows of x out of the exchange.  Row j (of n_rows <= 4) is 512 tagged words starting at exchange
+  // word rw[j]; its values go to the stage at byte rd[j] as fp16, in the permuted unit order of batch
+  // row rm[j].  Every lane fetches the 8 words of one unit, again and again until every word of
+  // every row carries this launch's tag -- then all of them have arrived, whatever else the
+  // producers still have in flight.  (These loads are the youngest: everything in the ring lands
+  // with them.)
+  auto fetch_tagged = [&](int n_rows, const int (&rw)[4], const int (&rd)[4], const int (&rm)[4], int src) {
+    const unsigned tag = lds_peek(&ctl->tag);
+    // nothing can have arrived from everywhere before this workgroup's own share has been stored
+    while (lds_peek(&ctl->stored) <= (unsigned)src && !lds_peek(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
+    const unsigned polls_allowed = spin_limit >> 4;  // (a poll here is a memory round trip, not a look at LDS)
+    unsigned polls = 0;
+    uint4_t t[4][2];
+    for (;;) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < n_rows) {
+          const unsigned *p = exchange + rw[j] + (lane ^ ((rm[j] ^ (lane >> 4)) & 3)) * 8;
+          asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(t[j][0]) : "v"(p) : "memory");
+          asm volatile("global_load_dwordx4 %0, %1, off offset:16 sc1" : "=v"(t[j][1]) : "v"(p) : "memory");
+        }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      unsigned bad = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (j < n_rows) {
+          asm volatile("" : "+v"(t[j][0]), "+v"(t[j][1]));  // (read below the wait)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bad |= (t[j][0][e] ^ tag) | (t[j][1][e] ^ tag);
+        }
+      if (__builtin_amdgcn_ballot_w64((bad >> 16) != 0u) == 0) break;
+      if (polls++ >= polls_allowed || lds_peek(&ctl->failed)) {  // some workgroup is not running: give up
+        if (lane == 0) {
+          __hip_atomic_store(&ctl->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if (status) atomicExch(status, 1);
+        }
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < n_rows) {
+        uint4_t q;  // the low halves of the eight words
+        q.x = __builtin_amdgcn_perm(t[j][0].y, t[j][0].x, 0x05040100u);
+        q.y = __builtin_amdgcn_perm(t[j][0].w, t[j][0].z, 0x05040100u);
+        q.z = __builtin_amdgcn_perm(t[j][1].y, t[j][1].x, 0x05040100u);
+        q.w = __builtin_amdgcn_perm(t[j][1].w, t[j][1].z, 0x05040100u);
+        asm volatile("ds_write_b128 %0, %1" : : "v"(x_rd + rd[j] + lane * 16), "v"(q) : "memory");
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
   // an entry whose x chunks do not fit the stage together fetches the chunk of its NEXT phase as
   // soon as the operands of the current one are in registers, instead of draining the ring for it
   int ahead_d = -1, ahead_chunk = -1;  // the stage holds (or will hold) this chunk of entry ahead_d
@@ -512,17 +620,39 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       x_loaded = nullptr;
       st_x = nullptr;
     }
+    // x out of the exchange (the host's plan: x is what entry x_src of this launch produces)
+    const int x_src = SINGLE ? -1 : (int)plan->x_src[d];
+    const int x_word = SINGLE ? -1 : plan->x_word[d];
+    if (x_src != x_from) {  // another producer: other values, even at the same address
+      x_loaded = nullptr;
+      st_x = nullptr;
+      x_from = x_src;
+    }
     // an entry with several phases whose x chunks all fit the stage fetches them in one go: one
     // drain of the ring per entry instead of one per phase
     const bool fits_all = phases > 1 && phases * m_rows * 1024 <= kStageBytes;
     bool staged = fits_all && st_x == x && st_k == k_in && st_m == m_rows;
     if (fits_all && !staged && nrb > 0) {
-      for (int phase = 0; phase < phases; ++phase) {
-        const int chunk = phase * kWaves + wave;
-        if (chunk * 512 >= k_in) continue;
-        for (int m = 0; m < m_rows; ++m)
-          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + x_unit(m),
-                                           xstage + (phase * m_rows + m) * 1024, 16, 0, kAuxDeviceCoherent);
+      if (x_word >= 0) {
+        int rw[4] = {0, 0, 0, 0}, rd[4] = {0, 0, 0, 0}, rm[4] = {0, 0, 0, 0}, n_rows = 0;
+        for (int phase = 0; phase < phases; ++phase) {
+          const int chunk = phase * kWaves + wave;
+          if (chunk * 512 >= k_in) continue;
+          for (int m = 0; m < m_rows; ++m, ++n_rows) {
+            rw[n_rows & 3] = x_word + m * k_in + chunk * 512;
+            rd[n_rows & 3] = (phase * m_rows + m) * 1024;
+            rm[n_rows & 3] = m;
+          }
+        }
+        fetch_tagged(n_rows, rw, rd, rm, x_src);
+      } else {
+        for (int phase = 0; phase < phases; ++phase) {
+          const int chunk = phase * kWaves + wave;
+          if (chunk * 512 >= k_in) continue;
+          for (int m = 0; m < m_rows; ++m)
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + x_unit(m),
+                                             xstage + (phase * m_rows + m) * 1024, 16, 0, kAuxDeviceCoherent);
+        }
       }
       wait_vm<0>();
       st_x = x;
@@ -549,6 +679,15 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
               else if (ahead_after == 2) wait_vm<2 * kItemOps>();
               else if (ahead_after == 1) wait_vm<kItemOps>();
               else wait_vm<0>();
+            } else if (x_word >= 0) {
+              int rw[4] = {0, 0, 0, 0}, rd[4] = {0, 0, 0, 0}, rm[4] = {0, 0, 0, 0};
+              for (int m = 0; m < m_rows; ++m) {
+                rw[m & 3] = x_word + m * k_in + chunk * 512;
+                rd[m & 3] = m * 1024;
+                rm[m & 3] = m;
+              }
+              fetch_tagged(m_rows, rw, rd, rm, x_src);
+              drained = true;
             } else {
               for (int m = 0; m < m_rows; ++m)
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + chunk * 512) + x_unit(m),
@@ -756,10 +895,9 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
 
 // (external linkage: the host takes its address for hipFuncSetAttribute)
 template <int MC, int NS>
-__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int first_entry, int *status,
-                                                                  unsigned *words, unsigned spin_limit) {
-  gemv_stream_body<MC, NS, false>(reinterpret_cast<const Entry *>(entries), n_entries, first_entry, status, words, spin_limit,
-                                  Entry{});
+__global__ __launch_bounds__(kThreadsAll) void gemv_stream_kernel(const void *entries, int n_entries, int *status, unsigned *words,
+                                                                  unsigned spin_limit, const SequencePlan plan) {
+  gemv_stream_body<MC, NS, false>(reinterpret_cast<const Entry *>(entries), n_entries, status, words, spin_limit, &plan, Entry{});
 }
 
 // one GEMV through the same body: what gq_gemv_f16 launches for large weights
@@ -778,7 +916,8 @@ __global__ __launch_bounds__(kThreadsAll) void gemv_stream_single_kernel(const g
   e.group_size = desc.group_size;
   e.wait_entries = 0;
   e.activation = desc.activation;
-  gemv_stream_body<MC, NS, true>(nullptr, 1, 0, nullptr, nullptr, 0u, e);  // (an entry without a wait touches no progress word)
+  // (an entry without a wait touches neither progress words nor exchange: no plan is read)
+  gemv_stream_body<MC, NS, true>(nullptr, 1, nullptr, nullptr, 0u, nullptr, e);
 }
 
 namespace {
@@ -863,6 +1002,90 @@ int launch_gemv_streamed(const uint16_t *x, int64_t m_rows, const uint16_t *pack
 
 int64_t gemv_sequence_workspace_bytes() { return (int64_t)kSequenceWords * 4; }
 
+namespace {
+
+bool overlap(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes) {
+  const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
+  return a0 < b0 + (uintptr_t)b_bytes && b0 < a0 + (uintptr_t)a_bytes;
+}
+
+// The plan of one launch (entries e[0..n), `first` entries of the sequence precede them and are
+// complete when the launch starts).
+//
+// Entry i reads its x through the exchange when x lies inside the results of an earlier entry p of
+// the launch (the latest one that writes any of it) and waiting for the tags is all the
+// synchronisation the entry needs:
+//   * it waits for nothing past p (wait_entries <= p + 1): once every workgroup has delivered its
+//     share of p, every workgroup has also finished reading the inputs of all entries up to p (a
+//     wave works through the entries in order), which is what a declared wait protects when
+//     buffers are re-used;
+//   * out_bias is not a result of this launch, and results of the launch that y overwrites were
+//     written with the same base and shape (then the same lane of the same workgroup wrote them, in
+//     program order);
+//   * the x chunks of a wave fit its stage at once (one phase, or all phases together), x starts
+//     on a 16-byte unit of the producer's results, and the exchange has room for the producer.
+// Any other entry that reads results of this launch (x or out_bias) waits for the reported
+// completion of their producer, whatever it declares: reported completion is what makes plain
+// loads see them.
+void plan_launch(const gq_gemv_desc *e, int n, int64_t first, SequencePlan &plan) {
+  bool tagged[kMaxEntries];
+  int64_t used_words = 0;
+  plan.uses_exchange = 0;
+  for (int i = 0; i < n; ++i) {
+    plan.ex_word[i] = plan.x_word[i] = -1;
+    plan.x_src[i] = -1;
+    tagged[i] = false;
+    const gq_gemv_desc &d = e[i];
+    int need = (int)(d.wait_entries > first ? d.wait_entries - first : 0);
+    const int64_t x_bytes = (int64_t)d.m_rows * d.k_in * 2, y_bytes = (int64_t)d.m_rows * d.n_out * 2;
+    int src = -1, bias_src = -1;
+    bool same_owner = true;
+    for (int j = i - 1; j >= 0; --j) {
+      const int64_t yj_bytes = (int64_t)e[j].m_rows * e[j].n_out * 2;
+      if (src < 0 && overlap(d.x, x_bytes, e[j].y, yj_bytes)) src = j;
+      if (bias_src < 0 && d.out_bias && overlap(d.out_bias, (int64_t)d.n_out * 2, e[j].y, yj_bytes)) bias_src = j;
+      if (overlap(d.y, y_bytes, e[j].y, yj_bytes) && !(e[j].y == d.y && e[j].n_out == d.n_out && e[j].m_rows == d.m_rows))
+        same_owner = false;
+    }
+    if (src >= 0) {
+      const gq_gemv_desc &p = e[src];
+      const int64_t off = (const char *)d.x - (const char *)p.y;
+      const int phases = (d.k_in + 4095) / 4096;
+      const bool fits = phases == 1 || (int64_t)phases * d.m_rows * 1024 <= kStageBytes;
+      tagged[i] = off >= 0 && off + x_bytes <= (int64_t)p.m_rows * p.n_out * 2 && off % 16 == 0 && fits && need <= src + 1 &&
+                  bias_src < 0 && same_owner;
+      if (tagged[i]) plan.x_src[i] = (int16_t)src;
+      else if (need < src + 1) need = src + 1;
+    }
+    if (bias_src >= 0 && need < bias_src + 1) need = bias_src + 1;
+    plan.need[i] = (int16_t)need;
+  }
+  // room in the exchange, in the order the producers run
+  for (int p = 0; p < n; ++p) {
+    bool wanted = false;
+    for (int i = p + 1; i < n && !wanted; ++i) wanted = tagged[i] && plan.x_src[i] == p;
+    if (!wanted) continue;
+    const int64_t words = ((int64_t)e[p].m_rows * e[p].n_out + 63) / 64 * 64;
+    if (used_words + words > kExchangeWords) continue;
+    plan.ex_word[p] = (int32_t)used_words;
+    used_words += words;
+    plan.uses_exchange = 1;
+  }
+  for (int i = 0; i < n; ++i) {
+    if (!tagged[i]) continue;
+    const int src = plan.x_src[i];
+    if (plan.ex_word[src] < 0) {  // no room: wait for the producer's reported completion instead
+      plan.x_src[i] = -1;
+      if (plan.need[i] < src + 1) plan.need[i] = (int16_t)(src + 1);
+      continue;
+    }
+    plan.need[i] = 0;
+    plan.x_word[i] = plan.ex_word[src] + (int32_t)(((const char *)e[i].x - (const char *)e[src].y) / 2);
+  }
+}
+
+}  // namespace
+
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
                          void *workspace, int64_t spin_limit, hipStream_t stream) {
   int max_m = 1;
@@ -917,8 +1140,9 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     }                                                                                                         \
     for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
       const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
-      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, (int)first, status,       \
-                                                                 words, spins);                               \
+      SequencePlan plan;                                                                                      \
+      plan_launch(host + first, n, first, plan);                                                              \
+      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status, words, spins, plan); \
     }                                                                                                         \
   } while (0)
   if (max_m <= 2) GQ_STREAM(2, 3);

@@ -607,14 +607,18 @@ def test_gemv_sequences_with_own_workspaces_on_two_streams(hip, device, oracle):
             x_prev = yy
 
 
+@pytest.mark.parametrize("next_input", ["o", "alternate"])
 @pytest.mark.parametrize("m_rows", [1, 4])
-def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows):
+def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows, next_input):
     """The schedule the layer-stack benchmark times, on three full-size layers with real data flowing
     through every declared wait: per layer the entries up (16384 x 4096, waits for the previous
     layer), fused qkv (12288 x 4096), down (4096 x 16384, waits for up), o (4096 x 4096, waits for
     qkv), every weight in the streaming layout.  up and qkv read the layer input, down reads up's
     output, o reads 4096-wide rows out of qkv's output, and the next layer's input is o's output
-    (even layers) or down's (odd layers).  Every entry is checked against the oracle applied to the
+    ("o": what the benchmark times; every result then travels through the kernel's tagged exchange)
+    or o's and down's in turn ("alternate": the entries that read down's output wait for more than
+    its producer, so they wait for reported completion, next to entries that use the exchange).
+    Every entry is checked against the oracle applied to the
     inputs the device had; then the same sequence with the buffers of a role shared by all layers
     (as the benchmark does: write-after-read hazards that only the declared waits resolve) must
     end with the same bits."""
@@ -656,7 +660,7 @@ def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows
             last = seq.add(v_rows(ys["qkv"]), w["o"][1], None, None, ys["o"], wait_for=qkv)
             plan += [(h, w["up"][0], ys["up"]), (h, w["qkv"][0], ys["qkv"]), (ys["up"], w["down"][0], ys["down"]),
                      (v_rows(ys["qkv"]), w["o"][0], ys["o"])]
-            h = ys["o"] if layer % 2 == 0 else ys["down"]
+            h = ys["o"] if layer % 2 == 0 or next_input == "o" else ys["down"]
         return seq, plan
 
     seq, plan = build(shared_buffers=False)
