@@ -264,7 +264,7 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     return r
 
 
-def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384):
+def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384, modes=None):
     """Benchmark configuration 5: 28 layers x {4 x [4096x4096], [16384x4096], [4096x16384]} as a
     sequence of fused GEMVs, every matrix distinct (3.17 GB of packed weight in total)."""
     import torch
@@ -292,14 +292,16 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
 
     results = {"m": m_rows, "entries": len(mats), "weight_bytes": w_bytes}
     # (1) one launch per matrix, replayed from a HIP graph
-    one_pass(stream_handle())
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    if modes is None:
         one_pass(stream_handle())
-    ms = time_launches(lambda _: graph.replay(), passes, warmup)
-    results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
-                                   "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS}
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            one_pass(stream_handle())
+        ms = time_launches(lambda _: graph.replay(), passes, warmup)
+        results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                                       "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
+                                       "roofline": hbm_roofline("gemv_mfma_kernel / gemv_stream_single_kernel (168 launches)", w_bytes, ms)}
     # (2) the whole stack as one gq_gemv_sequence_f16 call, with the dependencies of a decoder layer
     # declared per entry.  Roles per layer, in `mats` order: q k v o up down.
     #   sequential block   q waits for the previous layer, k and v share its input, then o, up and
@@ -406,6 +408,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                        ("sequence_decoder_data_flow", lambda seq: data_flow(seq, streaming=False)),
                        ("sequence_decoder_data_flow_streaming_layout", data_flow),
                        ("sequence_no_waits", free), ("sequence_no_waits_streaming_layout", free_streaming)):
+        if modes is not None and mode not in modes:
+            continue
         seq = hip.GemvSequence(device)
         fill(seq)
         for y in ys + [y_qkv] + y_o2:
@@ -435,8 +439,6 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         results[mode]["max_error_vs_single_call"] = worst
         if not worst <= 2e-3 or results[mode]["status"] != 0:
             raise SystemExit(f"bench.py: stack mode {mode} (m={m_rows}) is wrong: error {worst}, status {results[mode]['status']}")
-    results["per_launch_graph"]["roofline"] = hbm_roofline("gemv_mfma_kernel / gemv_stream_single_kernel (168 launches)", w_bytes,
-                                                           results["per_launch_graph"]["us_per_pass"] / 1e3)
     return results
 
 

@@ -126,6 +126,11 @@ static_assert(sizeof(CachedEntry) == 64, "entry cache layout");
 // agent-scope atomic load; it pairs with the agent-scope stores of y and of the progress words
 // (sc0 | sc1, system scope, costs another 2 % of a pass)
 constexpr int kAuxDeviceCoherent = 1 << 4;
+// cache policy of the weight loads (read once)
+#ifndef GQ_WEIGHT_AUX
+#define GQ_WEIGHT_AUX 0
+#endif
+constexpr int kAuxWeights = GQ_WEIGHT_AUX;
 
 // LDS words shared by the waves of a workgroup
 struct Control {
@@ -477,24 +482,24 @@ __device__ __forceinline__ void gemv_stream_body(const Entry *__restrict__ entri
       const char *blk = pe.packed + ((int64_t)rb * (pe.k_in >> 9) + chunk) * kItemBytes + lane * 16;
 #pragma unroll
       for (int s = 0; s < 4; ++s)
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + s * 1024), dst + s * 1024, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + s * 1024), dst + s * 1024, 16, 0, kAuxWeights);
       // (two loads of 256 bytes, like the other layout: every item counts kItemOps loads)
-      if (kc == 0) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, 0);
-      if (kc == 1) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, 0);
+      if (kc == 0) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, kAuxWeights);
+      if (kc == 1) __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(blk + 4096), dst + 4096, 16, 0, kAuxWeights);
       return;
     }
     const char *src = pe.packed + (int64_t)rb * 16 * (pe.k_in >> 1) + chunk * 256;
     const uint32_t off = (uint32_t)row * (uint32_t)(pe.k_in >> 1) + (uint32_t)kc * 16u;
 #pragma unroll
     for (int s = 0; s < 4; ++s)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(src + off + s * 64), dst + s * 1024, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(src + off + s * 64), dst + s * 1024, 16, 0, kAuxWeights);
     // lanes 0..15 fetch the 8 scales of their row's chunk, lanes 16..31 the 8 biases
     const uint32_t off2 = (uint32_t)row * (uint32_t)(pe.k_in >> 5);
     const int64_t base2 = (int64_t)rb * 16 * (pe.k_in >> 5) + chunk * 16;
     if (kc == 0)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.scale + base2 + off2), dst + 4096, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.scale + base2 + off2), dst + 4096, 16, 0, kAuxWeights);
     if (kc == 1)
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.bias + base2 + off2), dst + 4096, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(pe.bias + base2 + off2), dst + 4096, 16, 0, kAuxWeights);
   };
 
   Cursor prod = {0, 0, 0, 0};  // the producer's position: first item of this wave
