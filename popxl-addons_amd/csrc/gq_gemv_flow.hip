@@ -1,0 +1,519 @@
+// The data-flow kernel of the GEMV sequence: a persistent kernel for launches whose weights are in
+// the streaming layout and whose dependencies all travel through the exchange (a decoder's layer
+// stack at batch 1 to 4).  The LDS-ring kernel of gq_gemv_stream.hip serves everything else.
+//
+// Why a second kernel: a stack of dependent GEMVs stalls at every layer boundary (the next layer
+// needs every output of this one), and a stall only costs nothing if the weights keep streaming
+// into a buffer meanwhile AND the arithmetic then catches up faster than memory delivers.  This
+// kernel is built for few instructions per byte: 16 waves per compute unit (four per SIMD), a work
+// unit of 16 weight rows x 256 input features (2304 bytes: three direct-to-LDS loads into a
+// four-deep ring per wave, 144 KiB per compute unit in flight or buffered, issued across entry
+// boundaries -- weights never depend on results), and no staging of x at all.
+//
+// Arithmetic (v_mfma_f32_16x16x32_f16, one per 512 weights).  B operand = raw codes: the nibble
+// or-ed into the mantissa of 64.0 or 1024.0, five VALU instructions per eight weights; the offsets
+// are taken out of the accumulator before the first product (it starts at -sum off_k x_k), scale
+// and bias are applied to GROUP SUMS.  A operand = x, laid out so that one accumulator separates the
+// four groups of a unit and up to four batch rows: A row i = (group g = i >> 2, batch row m = i & 3)
+// holds x[m] on the 64 features of group g and zero elsewhere.  The two 1 KiB loads of a unit
+// (128 features each) share their four A registers and have an accumulator each; a row is valid
+// in the accumulator of the load its group lies in.  Lane (n, kc) -- weight row n, 32-feature
+// slice kc -- finds in the accumulator registers e the rows 4 kc + e = (group kc, batch row e): the
+// group whose scale and bias it reads as two 16-bit LDS loads.  sum x and sum off x per row come
+// out of eight MFMAs against constant B operands, in the same registers.
+//
+// x comes straight from memory into the A registers: 64 contiguous bytes per active lane, 8 lanes
+// per batch row.  Results that a later entry of the launch reads travel through the exchange in
+// the form the consumer wants: the fp16 bits of -y (zero as -0.0: an all-zero word means "not
+// written yet"; the sign is taken out again where the sums leave the wave), eight at a time in the
+// order (0,4,1,5,2,6,3,7) in which the raw codes of a 32-bit word come out.  A wave polls exactly
+// the 256 features it multiplies, so a dependency is between 16 producing workgroups and one wave,
+// not a barrier of the device; nothing is reported, counted or flushed.
+#include "gq_gemv_sequence.h"
+
+namespace gq {
+namespace {
+
+constexpr int kFlowWaves = 16;
+constexpr int kFlowThreads = kFlowWaves * 64;
+constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
+constexpr int kFlowPR = 4;              // row blocks per pass (their running sums stay in registers)
+// ring slots per wave and sets of mailboxes, by batch capacity (160 KiB of LDS)
+constexpr int flow_depth(int mc) { return mc == 4 ? 3 : 4; }
+constexpr int flow_sets(int mc) { return mc == 2 ? 1 : 2; }
+
+struct FlowEntry {  // what the work loop needs of an entry, in LDS
+  const char *blob;
+  const half_t *x, *out_bias;
+  half_t *y;
+  int n_out, k_in;
+  int x_word, ex_word;  // where x starts in the exchange (-1: in memory at x); where the results go (-1: nowhere)
+  short x_src, nrb;     // producer of x in this launch (-1: none); row blocks of this workgroup
+  char m_rows, act;
+  short pad;
+};
+static_assert(sizeof(FlowEntry) == 56, "entry cache layout");
+
+struct FlowControl {
+  unsigned deposited[2];  // mailbox deposits into the set since it was last emptied
+  unsigned reduced[2];    // reductions done on the set
+  unsigned failed;        // a wave gave up waiting
+  unsigned stored;        // entries whose results this workgroup has stored (stores issued)
+  unsigned waves_done;
+  unsigned half;          // the half of the exchange this launch uses
+};
+
+template <int MC>
+constexpr int flow_lds_bytes() {
+  return kFlowWaves * flow_depth(MC) * kUnitBytes + kMaxEntries * (int)sizeof(FlowEntry) +
+         flow_sets(MC) * kFlowWaves * kFlowPR * MC * 16 * 4 + 64;
+}
+
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+
+// raw_codes() of the other kernel without inline assembly: the compiler's hazard recogniser does
+// not look into assembly -- here only part of an accumulator is live at batch 1, the register
+// allocator re-uses the rest for the next B operand, and a VALU write to a register that an MFMA in
+// flight is still going to write needs wait states that only the compiler can place.  The masks
+// and magic numbers come in vector registers the compiler cannot see through, which is what makes
+// it select v_and_or_b32 (as literals they would cost a v_and and a v_or each).
+__device__ __forceinline__ half8_t raw_codes_c(uint32_t w, uint32_t mask_lo, uint32_t mask_hi, uint32_t magic_lo,
+                                               uint32_t magic_hi) {
+  const uint32_t hi = w >> 8;
+  uint4_t v;
+  v.x = (hi & mask_hi) | magic_hi;  // codes 0, 4: 64 + c
+  v.y = (hi & mask_lo) | magic_lo;  // codes 1, 5: 1024 + c
+  v.z = (w & mask_hi) | magic_hi;   // codes 2, 6: 64 + c
+  v.w = (w & mask_lo) | magic_lo;   // codes 3, 7: 1024 + c
+  return __builtin_bit_cast(half8_t, v);
+}
+
+template <int MC>
+__device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int n_entries, int *__restrict__ status,
+                                          unsigned *words, unsigned spin_limit, const SequencePlan *plan) {
+  constexpr int D = flow_depth(MC), S = flow_sets(MC), PR = kFlowPR;
+  constexpr int kMail = PR * MC * 16;  // floats a wave deposits per pass: [row block][m][n]
+  extern __shared__ __attribute__((aligned(64))) char lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = uni(tid >> 6);
+  const int n = lane & 15, kc = lane >> 4;
+  const int G = gridDim.x, b = blockIdx.x;
+  char *const ring = lds + wave * (D * kUnitBytes);
+  FlowEntry *const cache = reinterpret_cast<FlowEntry *>(lds + kFlowWaves * D * kUnitBytes);
+  float *const mail = reinterpret_cast<float *>(lds + kFlowWaves * D * kUnitBytes + kMaxEntries * sizeof(FlowEntry));
+  FlowControl *const ctl = reinterpret_cast<FlowControl *>(mail + S * kFlowWaves * kMail);
+
+  for (int i = tid; i < n_entries; i += kFlowThreads) {
+    const Entry e = entries[i];
+    FlowEntry c;
+    c.blob = reinterpret_cast<const char *>(e.packed);
+    c.x = e.x;
+    c.out_bias = e.out_bias;
+    c.y = e.y;
+    c.n_out = e.n_out;
+    c.k_in = e.k_in;
+    c.x_word = plan->x_word[i];
+    c.ex_word = plan->ex_word[i];
+    c.x_src = plan->x_src[i];
+    const int rb = (e.n_out + 15) >> 4;
+    c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
+    c.m_rows = (char)e.m_rows;
+    c.act = (char)e.activation;
+    c.pad = 0;
+    cache[i] = c;
+  }
+  if (tid == 0) {
+    const unsigned epoch = __hip_atomic_load(words + kFlowEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *ctl = FlowControl{{0u, 0u}, {0u, 0u}, 0u, 0u, 0u, epoch & 1u};
+  }
+  __syncthreads();
+  const unsigned half = (unsigned)uni((int)ctl->half);
+  unsigned short *const ex_all = reinterpret_cast<unsigned short *>(words + kFlowExchangeWord);
+  unsigned short *const ex16 = ex_all + (size_t)half * kFlowHalfValues;
+  {
+    // what the launch before this one left in the other half (that launch is complete; the one after
+    // this one, which will use that half, starts when these stores are)
+    const unsigned dirty = __hip_atomic_load(words + kFlowExtentWord + (1u - half), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint4_t *other = reinterpret_cast<uint4_t *>(ex_all + (size_t)(1u - half) * kFlowHalfValues);
+    for (unsigned i = (unsigned)b * kFlowThreads + tid; i < dirty / 8; i += (unsigned)G * kFlowThreads)
+      other[i] = uint4_t{0u, 0u, 0u, 0u};
+  }
+  // (nothing the compiler knows of is pending when the work loop starts: it would guard registers
+  // against those loads on every trip, with a wait for ALL loads of the ring)
+  wait_vm<0>();
+
+  // ---- lane constants
+  const uint32_t ring_rd = (uint32_t)(uintptr_t)ring;
+  const uint32_t lane16 = (uint32_t)lane * 16u;
+  const int hpar = wave & 1;  // which half of a 4608-byte block of the streaming layout this wave's units are
+  // the scales and biases of a unit: lanes 0..31 fetch the 32-bit words (row l >> 1, pair l & 1) of the
+  // block's scales that belong to this half, lanes 32..63 those of its biases (the instruction
+  // adds its offset, 2048, to both the address and the place in the slot)
+  const uint32_t sb_fetch = 2048u - hpar * 2048u + (uint32_t)(lane >> 5) * 256u + (uint32_t)((lane & 31) >> 1) * 16u + hpar * 8u +
+                            (uint32_t)(lane & 1) * 4u;
+  // ... and where lane (n, kc) finds the scale of (row n, group kc) among them; its bias 128 bytes on
+  const uint32_t sb_read = (uint32_t)(2 * n + (kc >> 1)) * 4u + (uint32_t)(kc & 1) * 2u;
+  uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u, kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
+  asm volatile("" : "+v"(kMaskLo), "+v"(kMaskHi), "+v"(kMagicLo), "+v"(kMagicHi));
+  // A row of this lane: group a_g of the unit, batch row a_m; its slice kc lies in that group or not
+  const int a_g = n >> 2, a_m = n & 3;
+  const bool a_match = (kc >> 1) == (a_g & 1);
+  const int a_off = a_g * 64 + (kc & 1) * 32;  // first feature (within the unit's 256) of this lane's 32
+
+  // ---- the producer: walks this wave's units D ahead of the consumer; all of it wave-uniform
+  struct Walk {
+    int d, pass, hcp, j;  // entry, pass of row blocks, this wave's how-manieth 256-feature piece, row block in pass
+    int nrb, n_hc, nj, chunks;
+    const char *blob;
+  };
+  auto enter = [&](Walk &w) {  // first unit of entry w.d (n_hc == 0 or nrb == 0: none)
+    w.pass = w.hcp = w.j = 0;
+    w.nrb = w.n_hc = w.nj = 0;
+    if (w.d >= n_entries) return;
+    w.nrb = uni(cache[w.d].nrb);
+    const int k_in = uni(cache[w.d].k_in);
+    w.chunks = k_in >> 9;
+    const int pieces = k_in >> 8;
+    w.n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
+    w.nj = min(PR, w.nrb);
+    w.blob = uni_ptr(cache[w.d].blob);
+  };
+  auto next_entry = [&](Walk &w) {
+    do {
+      ++w.d;
+      enter(w);
+    } while (w.d < n_entries && (w.n_hc == 0 || w.nrb == 0));
+  };
+  auto advance = [&](Walk &w) {
+    if (++w.j < w.nj) return;
+    w.j = 0;
+    if (++w.hcp < w.n_hc) return;
+    w.hcp = 0;
+    ++w.pass;
+    w.nj = min(PR, w.nrb - w.pass * PR);
+    if (w.nj > 0) return;
+    next_entry(w);
+  };
+  auto issue = [&](const Walk &w, int slot) {
+    const int64_t block = (int64_t)(b + (w.pass * PR + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
+    const char *src = w.blob + block * (2 * kUnitBytes) + hpar * 2048;
+    const uint32_t dst = ring_rd + (uint32_t)slot * kUnitBytes;
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %3\n\t"
+        "global_load_lds_dwordx4 %1, %3 offset:1024\n\t"
+        "global_load_lds_dword %2, %3 offset:2048"
+        :
+        : "s"(dst), "v"(lane16), "v"(sb_fetch), "s"(src)
+        : "memory");
+  };
+
+  Walk prod;
+  prod.d = -1;
+  prod.blob = nullptr;
+  prod.chunks = 0;
+  next_entry(prod);
+  int ahead = 0;  // units issued and not yet consumed
+  while (ahead < D && prod.d < n_entries) {
+    issue(prod, ahead);
+    ++ahead;
+    advance(prod);
+  }
+  int slot = 0;    // ring slot of the consumer's unit
+  unsigned q = 0;  // passes so far (the same count in every wave)
+
+  // ---- the A registers and what they hold
+  half8_t xa[4];
+  float4_t negcorr = {0.f, 0.f, 0.f, 0.f}, xsum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) xa[w] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  const half_t *xa_x = nullptr;
+  int xa_word = -2, xa_src = -2, xa_k = 0, xa_m = 0, xa_hc = -1;
+
+  auto give_up = [&]() {
+    if (lane == 0) {
+      __hip_atomic_store(&ctl->failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (status) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
+
+  // x of (entry, piece hc) into the A registers.  These loads are the youngest of the wave:
+  // everything in its ring lands with them.
+  auto build = [&](const half_t *x, int x_word, int x_src, int k_in, int m_rows, int hc) {
+    const bool active = a_match && a_m < m_rows;
+    const int64_t at = (int64_t)a_m * k_in + hc * 256 + a_off;
+    uint4_t t[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) t[w] = uint4_t{0u, 0u, 0u, 0u};
+    if (x_word >= 0) {
+      // nothing can have arrived from everywhere before this workgroup's own share (if it has one) is stored
+      if (uni(cache[x_src].nrb) > 0)
+        while (lds_load(&ctl->stored) <= (unsigned)x_src && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
+      const unsigned short *p = ex16 + x_word + at;
+      const unsigned polls_allowed = spin_limit >> 4;  // (a poll is a memory round trip)
+      unsigned polls = 0;
+      for (;;) {
+        if (active) {
+          asm volatile(
+              "global_load_dwordx4 %0, %4, off sc1\n\t"
+              "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
+              "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
+              "global_load_dwordx4 %3, %4, off offset:48 sc1"
+              : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
+              : "v"(p)
+              : "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
+        // a value that has not arrived is a zero half-word
+        ushort2_t lo = __builtin_bit_cast(ushort2_t, t[0][0]);
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ushort2_t, t[w][c]));
+        const bool missing = active && (lo[0] == 0 || lo[1] == 0);
+        if (__builtin_amdgcn_ballot_w64(missing) == 0) break;
+        if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {  // some workgroup is not running: give up
+          give_up();
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
+    } else {
+      const half_t *p = x + at;
+      if (active) {
+        asm volatile(
+            "global_load_dwordx4 %0, %4, off sc1\n\t"
+            "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
+            "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
+            "global_load_dwordx4 %3, %4, off offset:48 sc1"
+            : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
+            : "v"(p)
+            : "memory");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
+      // the form of the exchange: sign flipped, eight at a time in the order of the raw codes
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        uint4_t f = t[w];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) f[c] ^= 0x80008000u;
+        t[w] = __builtin_bit_cast(uint4_t, permute_x(f));
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 4; ++w) xa[w] = __builtin_bit_cast(half8_t, t[w]);
+    // per A row: -sum off_k x_k (where every accumulator starts) and sum x_k, off = 64 or 1024 as the
+    // raw codes of a word come out: (64 + c, 64 + c, 1024 + c, 1024 + c) twice
+    const half8_t neg_off = {(half_t)-64.f, (half_t)-64.f, (half_t)-1024.f, (half_t)-1024.f,
+                             (half_t)-64.f, (half_t)-64.f, (half_t)-1024.f, (half_t)-1024.f};
+    const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+    negcorr = float4_t{0.f, 0.f, 0.f, 0.f};
+    xsum = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      negcorr = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], neg_off, negcorr, 0, 0, 0);
+      xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], ones, xsum, 0, 0, 0);
+    }
+  };
+
+  // one unit: ring slot -> registers -> 8 MFMAs -> this lane's group sums into tot
+  auto consume = [&](int s, float (&tot)[MC]) {
+    const uint32_t at = ring_rd + (uint32_t)s * kUnitBytes;
+    uint4_t w0, w1;
+    uint32_t sc, bi;
+    asm volatile(
+        "ds_read_b128 %0, %4\n\t"
+        "ds_read_b128 %1, %4 offset:1024\n\t"
+        "ds_read_u16 %2, %5 offset:2048\n\t"
+        "ds_read_u16 %3, %5 offset:2176\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(w0), "=&v"(w1), "=&v"(sc), "=&v"(bi)
+        : "v"(at + lane16), "v"(at + sb_read)
+        : "memory");
+    float4_t acc0 = negcorr, acc1 = negcorr;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], raw_codes_c(w0[w], kMaskLo, kMaskHi, kMagicLo, kMagicHi), acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], raw_codes_c(w1[w], kMaskLo, kMaskHi, kMagicLo, kMagicHi), acc1, 0, 0, 0);
+    }
+    const float scale = (float)__builtin_bit_cast(half_t, (unsigned short)sc);
+    const float bias = (float)__builtin_bit_cast(half_t, (unsigned short)bi);
+#pragma unroll
+    for (int e = 0; e < MC; ++e) {
+      const float sum = (kc & 2) ? acc1[e] : acc0[e];
+      tot[e] = __builtin_fmaf(scale, sum, __builtin_fmaf(bias, xsum[e], tot[e]));
+    }
+  };
+
+  // ---- the consumer
+  for (int d = 0; d < n_entries; ++d) {
+    const int nrb = uni(cache[d].nrb);
+    if (nrb == 0) continue;
+    const int k_in = uni(cache[d].k_in), m_rows = uni(cache[d].m_rows);
+    const int pieces = k_in >> 8;
+    const int n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
+    const int active_waves = min(kFlowWaves, pieces);
+    const half_t *x = reinterpret_cast<const half_t *>(uni_ptr(cache[d].x));
+    const int x_word = uni(cache[d].x_word), x_src = uni(cache[d].x_src);
+    for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
+      if (n_hc == 0) continue;
+      const int nj = min(PR, nrb - pass * PR);
+      float tot[PR][MC];
+#pragma unroll
+      for (int j = 0; j < PR; ++j)
+#pragma unroll
+        for (int e = 0; e < MC; ++e) tot[j][e] = 0.f;
+      for (int hcp = 0; hcp < n_hc; ++hcp) {
+        const int hc = wave + kFlowWaves * hcp;
+        if (!(xa_x == x && xa_word == x_word && xa_src == x_src && xa_k == k_in && xa_m == m_rows && xa_hc == hc)) {
+          build(x, x_word, x_src, k_in, m_rows, hc);
+          xa_x = x;
+          xa_word = x_word;
+          xa_src = x_src;
+          xa_k = k_in;
+          xa_m = m_rows;
+          xa_hc = hc;
+        }
+#pragma unroll
+        for (int j = 0; j < PR; ++j) {
+          if (j >= nj) break;
+          // the unit's three loads have landed when at most those of the D - 1 units after it are out
+          if (ahead == D) wait_vm<3 * (D - 1)>();
+          else wait_vm<0>();
+          consume(slot, tot[j]);
+          if (prod.d < n_entries) {
+            issue(prod, slot);
+            advance(prod);
+          } else {
+            --ahead;
+          }
+          slot = slot + 1 == D ? 0 : slot + 1;
+        }
+      }
+      // ---- the pass is done for this wave: its sums go to the mailbox; the wave that completes the
+      // set adds the waves' sums up and stores the results
+      const unsigned set = q % S, use = q / S;
+      float out[PR][MC];
+#pragma unroll
+      for (int j = 0; j < PR; ++j)
+#pragma unroll
+        for (int e = 0; e < MC; ++e) {
+          float v = tot[j][e];
+          v += lane_read(v, lane ^ 16);
+          v += lane_read(v, lane ^ 32);
+          out[j][e] = v;
+        }
+      while (lds_load(&ctl->reduced[set]) < use) __builtin_amdgcn_s_sleep(1);  // the set has been emptied
+      float *box = mail + (set * kFlowWaves + wave) * kMail;
+      if (kc == 0) {
+#pragma unroll
+        for (int j = 0; j < PR; ++j)
+          if (j < nj) {
+#pragma unroll
+            for (int e = 0; e < MC; ++e) box[(j * MC + e) * 16 + n] = out[j][e];
+          }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      unsigned before = 0;
+      if (lane == 0) before = __hip_atomic_fetch_add(&ctl->deposited[set], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      before = (unsigned)uni((int)before);
+      if (before + 1u != (unsigned)active_waves) continue;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      {
+        const int n_out = uni(cache[d].n_out), act = uni(cache[d].act), ex_word = uni(cache[d].ex_word);
+        unsigned short *y = reinterpret_cast<unsigned short *>(const_cast<char *>(uni_ptr(cache[d].y)));
+        const half_t *out_bias = reinterpret_cast<const half_t *>(uni_ptr(cache[d].out_bias));
+        const float *set_mail = mail + set * kFlowWaves * kMail;
+        for (int t = lane; t < nj * MC * 16; t += 64) {
+          const int n16 = t & 15, m = (t >> 4) % MC, j = t / (16 * MC);
+          float sum = 0.f;
+          for (int w = 0; w < active_waves; ++w) sum += set_mail[w * kMail + t];
+          sum = -sum;  // (the A registers hold -x)
+          const int row = (b + (pass * PR + j) * G) * 16 + n16;
+          if (m < m_rows && row < n_out) {
+            if (out_bias) sum += (float)out_bias[row];
+            const unsigned short hv = __builtin_bit_cast(unsigned short, (half_t)apply_activation(sum, act));
+            const int64_t flat = (int64_t)m * n_out + row;
+            __hip_atomic_store(y + flat, hv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (ex_word >= 0) {
+              // -y, zero as -0.0; value 8 q + e at place 8 q + (0,2,4,6,1,3,5,7)[e]
+              const unsigned short neg = (hv & 0x7FFFu) == 0 ? (unsigned short)0x8000u : (unsigned short)(hv ^ 0x8000u);
+              const int e8 = (int)(flat & 7);
+              const int64_t place = (flat & ~(int64_t)7) + ((e8 & 3) * 2 + (e8 >> 2));
+              __hip_atomic_store(ex16 + ex_word + place, neg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // (the mailbox reads are done)
+        if (lane == 0) {
+          __hip_atomic_store(&ctl->deposited[set], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          __hip_atomic_store(&ctl->reduced[set], use + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+          if ((pass + 1) * PR >= nrb)  // the entry's last pass in this workgroup
+            // (a maximum: the wave that completes the next entry's set may get here first)
+            __hip_atomic_fetch_max(&ctl->stored, (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    }
+  }
+  wait_vm<0>();  // no load may land in LDS after this workgroup has gone
+
+  // ---- the last wave of the last workgroup turns the exchange over: the next launch uses the other half
+  unsigned done = 0;
+  if (lane == 0) done = __hip_atomic_fetch_add(&ctl->waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  if ((unsigned)uni((int)done) != kFlowWaves - 1) return;
+  unsigned last = 0;
+  if (lane == 0) last = atomicAdd(words + kFlowExitedWord, 1u) == (unsigned)G - 1;
+  if (!uni((int)last)) return;
+  if (lane == 0) {
+    __hip_atomic_store(words + kFlowExtentWord + half, (unsigned)plan->exchange_values, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(words + kFlowExtentWord + (1u - half), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(words + kFlowEpochWord, half ^ 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(words + kFlowExitedWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+}  // namespace
+
+template <int MC>
+__global__ __launch_bounds__(kFlowThreads) void gemv_flow_kernel(const void *entries, int n_entries, int *status,
+                                                                 unsigned *words, unsigned spin_limit,
+                                                                 const SequencePlan plan) {
+  flow_body<MC>(reinterpret_cast<const Entry *>(entries), n_entries, status, words, spin_limit, &plan);
+}
+
+// Can this launch run on the data-flow kernel?  Every weight in the streaming layout, at most four
+// batch rows, and no entry that has to wait for reported completion.
+bool flow_eligible(const gq_gemv_desc *e, int n, const SequencePlan &plan) {
+  for (int i = 0; i < n; ++i)
+    if (e[i].scale != nullptr || e[i].bias != nullptr || e[i].m_rows > 4 || plan.need[i] != 0 || e[i].k_in % 512 != 0) return false;
+  return true;
+}
+
+int launch_flow(const gq_gemv_desc *host, const gq_gemv_desc *device, int n, int *status, unsigned *words, unsigned spins,
+                const SequencePlan &plan, int grid, int dev, hipStream_t stream) {
+  constexpr int kMaxDevices = 64;
+  if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
+  int max_m = 1;
+  for (int i = 0; i < n; ++i) max_m = host[i].m_rows > max_m ? host[i].m_rows : max_m;
+#define GQ_FLOW(MC)                                                                                           \
+  do {                                                                                                        \
+    constexpr int lds_bytes = flow_lds_bytes<MC>();                                                           \
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
+    static bool configured[kMaxDevices] = {false};                                                            \
+    if (!configured[dev]) {                                                                                   \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_flow_kernel<MC>),          \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);        \
+      if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
+      configured[dev] = true;                                                                                 \
+    }                                                                                                         \
+    gemv_flow_kernel<MC><<<dim3(grid), dim3(kFlowThreads), lds_bytes, stream>>>(device, n, status, words, spins, plan); \
+  } while (0)
+  if (max_m == 1) GQ_FLOW(1);
+  else if (max_m == 2) GQ_FLOW(2);
+  else GQ_FLOW(4);
+#undef GQ_FLOW
+  return GQ_OK;
+}
+
+}  // namespace gq

@@ -261,9 +261,11 @@ def test_gemv_sequence_chained_entries(hip, device, oracle, m_rows):
 
 @pytest.mark.parametrize("m_rows,chained", [(1, False), (2, False), (4, False), (1, True), (4, True)])
 def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
-    """Weights in the streaming layout of gq_gemv_prepack_f16 give bit for bit what the same
-    sequence gives on the three variables (same arithmetic, other addresses), with ragged row
-    counts, waits, and both layouts mixed in one sequence."""
+    """Weights in the streaming layout of gq_gemv_prepack_f16 give what the same sequence gives on
+    the three variables, with ragged row counts, waits, and both layouts mixed in one sequence.
+    Another kernel runs them when the whole launch is in the streaming layout (fp32 sums taken in
+    another order): the two agree to a few fp16 roundings, not bit for bit; a chain of entries
+    carries the difference of its inputs along."""
     from popxl_addons._gq_hip import GemvSequence, GQHipError, prepack_gemv
 
     if chained:
@@ -292,7 +294,9 @@ def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
             assert int(seq.status.item()) == 0 and int(seq2.status.item()) == 0
             for i, (y, y2) in enumerate(zip(outs, outs2)):
                 assert torch.isfinite(y2).all(), i
-                assert torch.equal(y, y2), (i, mixed)
+                top = y.float().abs().max().item()
+                worst = (y.float() - y2.float()).abs().max().item()
+                assert worst <= (4e-3 if chained else 1.5e-3) * top, (i, mixed, worst / top)
         if not chained:
             for y2, ref in zip(outs2, refs):
                 assert_close(y2.cpu().numpy(), ref)

@@ -72,7 +72,7 @@ def test_abi_version_and_error_text_without_gpu():
         _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 16384, 4096, 64, 0, 256, need - 1, None)
     assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE and "workspace" in str(e.value)
     # the sequence with a caller-owned workspace
-    assert lib.gq_gemv_sequence_workspace_bytes() == (256 + 4) * 128 + (16 << 20)  # progress lines, 3 words, 16 MiB exchange
+    assert lib.gq_gemv_sequence_workspace_bytes() == (256 + 4 + 4) * 128 + (32 << 20)  # progress lines, 3 + 4 words, two 16 MiB exchanges
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_gemv_sequence_ws_f16", 16, 16, 1, None, None, 0, 0, None)
     assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER and "workspace" in str(e.value)
