@@ -38,8 +38,13 @@ constexpr int kFlowWaves = 16;
 constexpr int kFlowThreads = kFlowWaves * 64;
 constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
 constexpr int kFlowPR = 4;              // row blocks per pass (their running sums stay in registers)
+// At batch 1 a ring slot also has room for the 256 values of x that its unit multiplies (512 bytes):
+// the producer fetches them with the first unit that needs them, ahead of time like the weights,
+// and in the order of the wave's loads they arrive before that unit -- no wait for x drains the ring.
+constexpr bool flow_x_in_slot(int mc) { return mc == 1; }
+constexpr int flow_slot_bytes(int mc) { return kUnitBytes + (flow_x_in_slot(mc) ? 512 : 0); }
 // ring slots per wave and sets of mailboxes, by batch capacity (160 KiB of LDS)
-constexpr int flow_depth(int mc) { return mc == 4 ? 3 : 4; }
+constexpr int flow_depth(int mc) { return mc == 2 ? 4 : 3; }
 constexpr int flow_sets(int mc) { return mc == 2 ? 1 : 2; }
 
 struct FlowEntry {  // what the work loop needs of an entry, in LDS
@@ -50,7 +55,7 @@ struct FlowEntry {  // what the work loop needs of an entry, in LDS
   int x_word, ex_word;  // where x starts in the exchange (-1: in memory at x); where the results go (-1: nowhere)
   short x_src, nrb;     // producer of x in this launch (-1: none); row blocks of this workgroup
   char m_rows, act;
-  short pad;
+  short x_id;           // the first entry of the launch that reads the same x (same values at the same place)
 };
 static_assert(sizeof(FlowEntry) == 56, "entry cache layout");
 
@@ -61,14 +66,20 @@ struct FlowControl {
   unsigned stored;        // entries whose results this workgroup has stored (stores issued)
   unsigned waves_done;
   unsigned half;          // the half of the exchange this launch uses
+  unsigned pad[8];
+  unsigned zeros[16];     // what the lanes of an A row without data read
 };
+static_assert(sizeof(FlowControl) == 128, "control block");
 
 template <int MC>
 constexpr int flow_lds_bytes() {
-  return kFlowWaves * flow_depth(MC) * kUnitBytes + kMaxEntries * (int)sizeof(FlowEntry) +
-         flow_sets(MC) * kFlowWaves * kFlowPR * MC * 16 * 4 + 64;
+  return kFlowWaves * flow_depth(MC) * flow_slot_bytes(MC) + kMaxEntries * (int)sizeof(FlowEntry) +
+         flow_sets(MC) * kFlowWaves * kFlowPR * MC * 16 * 4 + (int)sizeof(FlowControl);
 }
 
+#ifndef GQ_FLOW_EXP
+#define GQ_FLOW_EXP 0  // (timing experiments: parts of the kernel switched off)
+#endif
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
 
 // raw_codes() of the other kernel without inline assembly: the compiler's hazard recogniser does
@@ -92,15 +103,17 @@ template <int MC>
 __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int n_entries, int *__restrict__ status,
                                           unsigned *words, unsigned spin_limit, const SequencePlan *plan) {
   constexpr int D = flow_depth(MC), S = flow_sets(MC), PR = kFlowPR;
+  constexpr bool XS = flow_x_in_slot(MC);
+  constexpr int kSlot = flow_slot_bytes(MC);
   constexpr int kMail = PR * MC * 16;  // floats a wave deposits per pass: [row block][m][n]
   extern __shared__ __attribute__((aligned(64))) char lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = uni(tid >> 6);
   const int n = lane & 15, kc = lane >> 4;
   const int G = gridDim.x, b = blockIdx.x;
-  char *const ring = lds + wave * (D * kUnitBytes);
-  FlowEntry *const cache = reinterpret_cast<FlowEntry *>(lds + kFlowWaves * D * kUnitBytes);
-  float *const mail = reinterpret_cast<float *>(lds + kFlowWaves * D * kUnitBytes + kMaxEntries * sizeof(FlowEntry));
+  char *const ring = lds + wave * (D * kSlot);
+  FlowEntry *const cache = reinterpret_cast<FlowEntry *>(lds + kFlowWaves * D * kSlot);
+  float *const mail = reinterpret_cast<float *>(lds + kFlowWaves * D * kSlot + kMaxEntries * sizeof(FlowEntry));
   FlowControl *const ctl = reinterpret_cast<FlowControl *>(mail + S * kFlowWaves * kMail);
 
   for (int i = tid; i < n_entries; i += kFlowThreads) {
@@ -119,12 +132,12 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
     c.m_rows = (char)e.m_rows;
     c.act = (char)e.activation;
-    c.pad = 0;
+    c.x_id = plan->x_id[i];
     cache[i] = c;
   }
   if (tid == 0) {
     const unsigned epoch = __hip_atomic_load(words + kFlowEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *ctl = FlowControl{{0u, 0u}, {0u, 0u}, 0u, 0u, 0u, epoch & 1u};
+    *ctl = FlowControl{{0u, 0u}, {0u, 0u}, 0u, 0u, 0u, epoch & 1u, {}, {}};
   }
   __syncthreads();
   const unsigned half = (unsigned)uni((int)ctl->half);
@@ -144,7 +157,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
 
   // ---- lane constants
   const uint32_t ring_rd = (uint32_t)(uintptr_t)ring;
-  const uint32_t lane16 = (uint32_t)lane * 16u;
+  const uint32_t lane16 = (uint32_t)lane * 16u, lane4 = (uint32_t)lane * 4u;
   const int hpar = wave & 1;  // which half of a 4608-byte block of the streaming layout this wave's units are
   // the scales and biases of a unit: lanes 0..31 fetch the 32-bit words (row l >> 1, pair l & 1) of the
   // block's scales that belong to this half, lanes 32..63 those of its biases (the instruction
@@ -160,11 +173,20 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   const bool a_match = (kc >> 1) == (a_g & 1);
   const int a_off = a_g * 64 + (kc & 1) * 32;  // first feature (within the unit's 256) of this lane's 32
 
+  // what lane (row i, slice kc) of the A operand reads of a unit's 512 bytes of x in a ring slot; a lane
+  // without data reads zeros
+  const uint32_t zeros_rd = (uint32_t)(uintptr_t)ctl->zeros;
+  const uint32_t xa_rd = kUnitBytes + (uint32_t)a_off * 2u;
+  const bool a_lane = a_match && a_m == 0;  // (x in the slot is batch 1 only)
+
   // ---- the producer: walks this wave's units D ahead of the consumer; all of it wave-uniform
   struct Walk {
     int d, pass, hcp, j;  // entry, pass of row blocks, this wave's how-manieth 256-feature piece, row block in pass
     int nrb, n_hc, nj, chunks;
     const char *blob;
+    // batch 1: the x the A registers would hold at this point of the walk, and where the entry's x is
+    int key_id, key_hc;
+    const char *xrow;
   };
   auto enter = [&](Walk &w) {  // first unit of entry w.d (n_hc == 0 or nrb == 0: none)
     w.pass = w.hcp = w.j = 0;
@@ -194,10 +216,38 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     if (w.nj > 0) return;
     next_entry(w);
   };
-  auto issue = [&](const Walk &w, int slot) {
+  // where the x of entry d starts, in the form the A operand wants or not
+  auto x_row = [&](int d) -> const char * {
+    const int x_word = uni(cache[d].x_word);
+    return x_word >= 0 ? reinterpret_cast<const char *>(ex16 + x_word) : uni_ptr(cache[d].x);
+  };
+  // piece hc of x into the x part of a ring slot (two loads of 256 bytes)
+  auto issue_x = [&](const char *xrow, int hc, int slot) {
+    const char *src = xrow + hc * 512;
+    const uint32_t dst = ring_rd + (uint32_t)slot * kSlot + kUnitBytes;
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dword %1, %2 sc1\n\t"
+        "global_load_lds_dword %1, %2 offset:256 sc1"
+        :
+        : "s"(dst), "v"(lane4), "s"(src)
+        : "memory");
+  };
+  auto issue = [&](Walk &w, int slot) {
+    if (XS) {
+      // the first unit that multiplies another piece of x brings it along: its loads are older than the unit's
+      const int id = uni(cache[w.d].x_id), hc = wave + kFlowWaves * w.hcp;
+      if (id != w.key_id || hc != w.key_hc) {
+        if (id != w.key_id) w.xrow = x_row(w.d);
+        w.key_id = id;
+        w.key_hc = hc;
+        issue_x(w.xrow, hc, slot);
+      }
+    }
     const int64_t block = (int64_t)(b + (w.pass * PR + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
     const char *src = w.blob + block * (2 * kUnitBytes) + hpar * 2048;
-    const uint32_t dst = ring_rd + (uint32_t)slot * kUnitBytes;
+    const uint32_t dst = ring_rd + (uint32_t)slot * kSlot;
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
         "s_nop 0\n\t"
@@ -213,6 +263,8 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   prod.d = -1;
   prod.blob = nullptr;
   prod.chunks = 0;
+  prod.key_id = prod.key_hc = -1;
+  prod.xrow = nullptr;
   next_entry(prod);
   int ahead = 0;  // units issued and not yet consumed
   while (ahead < D && prod.d < n_entries) {
@@ -230,6 +282,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   for (int w = 0; w < 4; ++w) xa[w] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
   const half_t *xa_x = nullptr;
   int xa_word = -2, xa_src = -2, xa_k = 0, xa_m = 0, xa_hc = -1;
+  int key_id = -1, key_hc = -1;  // batch 1
 
   auto give_up = [&]() {
     if (lane == 0) {
@@ -237,74 +290,30 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
       if (status) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   };
-
-  // x of (entry, piece hc) into the A registers.  These loads are the youngest of the wave:
-  // everything in its ring lands with them.
-  auto build = [&](const half_t *x, int x_word, int x_src, int k_in, int m_rows, int hc) {
-    const bool active = a_match && a_m < m_rows;
-    const int64_t at = (int64_t)a_m * k_in + hc * 256 + a_off;
-    uint4_t t[4];
+  // a value that has not arrived is a zero half-word
+  auto any_missing = [&](const uint4_t (&t)[4], bool active) {
+    ushort2_t lo = __builtin_bit_cast(ushort2_t, t[0][0]);
 #pragma unroll
-    for (int w = 0; w < 4; ++w) t[w] = uint4_t{0u, 0u, 0u, 0u};
-    if (x_word >= 0) {
-      // nothing can have arrived from everywhere before this workgroup's own share (if it has one) is stored
-      if (uni(cache[x_src].nrb) > 0)
-        while (lds_load(&ctl->stored) <= (unsigned)x_src && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
-      const unsigned short *p = ex16 + x_word + at;
-      const unsigned polls_allowed = spin_limit >> 4;  // (a poll is a memory round trip)
-      unsigned polls = 0;
-      for (;;) {
-        if (active) {
-          asm volatile(
-              "global_load_dwordx4 %0, %4, off sc1\n\t"
-              "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
-              "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
-              "global_load_dwordx4 %3, %4, off offset:48 sc1"
-              : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
-              : "v"(p)
-              : "memory");
-        }
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
-        // a value that has not arrived is a zero half-word
-        ushort2_t lo = __builtin_bit_cast(ushort2_t, t[0][0]);
+    for (int w = 0; w < 4; ++w)
 #pragma unroll
-        for (int w = 0; w < 4; ++w)
+      for (int c = 0; c < 4; ++c) lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ushort2_t, t[w][c]));
+    return __builtin_amdgcn_ballot_w64(active && (lo[0] == 0 || lo[1] == 0)) != 0;
+  };
+  // x in memory order -> the form of the exchange: sign flipped, eight at a time in the order of the raw codes
+  auto to_exchange_form = [&](uint4_t (&t)[4]) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) lo = __builtin_elementwise_min(lo, __builtin_bit_cast(ushort2_t, t[w][c]));
-        const bool missing = active && (lo[0] == 0 || lo[1] == 0);
-        if (__builtin_amdgcn_ballot_w64(missing) == 0) break;
-        if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {  // some workgroup is not running: give up
-          give_up();
-          break;
-        }
-        __builtin_amdgcn_s_sleep(2);
-      }
-    } else {
-      const half_t *p = x + at;
-      if (active) {
-        asm volatile(
-            "global_load_dwordx4 %0, %4, off sc1\n\t"
-            "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
-            "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
-            "global_load_dwordx4 %3, %4, off offset:48 sc1"
-            : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
-            : "v"(p)
-            : "memory");
-      }
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
-      // the form of the exchange: sign flipped, eight at a time in the order of the raw codes
+    for (int w = 0; w < 4; ++w) {
+      uint4_t f = t[w];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        uint4_t f = t[w];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) f[c] ^= 0x80008000u;
-        t[w] = __builtin_bit_cast(uint4_t, permute_x(f));
-      }
+      for (int c = 0; c < 4; ++c) f[c] ^= 0x80008000u;
+      t[w] = __builtin_bit_cast(uint4_t, permute_x(f));
     }
+  };
+  // per A row: -sum off_k x_k (where every accumulator starts) and sum x_k, off = 64 or 1024 as the
+  // raw codes of a word come out: (64 + c, 64 + c, 1024 + c, 1024 + c) twice
+  auto finish_build = [&](const uint4_t (&t)[4]) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) xa[w] = __builtin_bit_cast(half8_t, t[w]);
-    // per A row: -sum off_k x_k (where every accumulator starts) and sum x_k, off = 64 or 1024 as the
-    // raw codes of a word come out: (64 + c, 64 + c, 1024 + c, 1024 + c) twice
     const half8_t neg_off = {(half_t)-64.f, (half_t)-64.f, (half_t)-1024.f, (half_t)-1024.f,
                              (half_t)-64.f, (half_t)-64.f, (half_t)-1024.f, (half_t)-1024.f};
     const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
@@ -316,22 +325,124 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
       xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], ones, xsum, 0, 0, 0);
     }
   };
+  // nothing can have arrived from everywhere before this workgroup's own share (if it has one) is stored
+  auto wait_own_share = [&](int x_src) {
+    if (uni(cache[x_src].nrb) > 0)
+      while (lds_load(&ctl->stored) <= (unsigned)x_src && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
+  };
 
-  // one unit: ring slot -> registers -> 8 MFMAs -> this lane's group sums into tot
-  auto consume = [&](int s, float (&tot)[MC]) {
-    const uint32_t at = ring_rd + (uint32_t)s * kUnitBytes;
+  // batch 1, a unit that brought x along found values that their producer had not delivered when
+  // they were fetched: fetch the piece again until it is complete (these loads are the youngest of
+  // the wave: everything in its ring lands with them)
+  auto refetch = [&](int s, int d, int hc, uint32_t xat, uint4_t (&t)[4]) {
+    wait_own_share(uni(cache[d].x_src));
+    const unsigned polls_allowed = spin_limit >> 4;  // (a poll is a memory round trip)
+    unsigned polls = 0;
+    for (;;) {
+      issue_x(x_row(d), hc, s);
+      wait_vm<0>();
+      asm volatile(
+          "ds_read_b128 %0, %4\n\t"
+          "ds_read_b128 %1, %4 offset:16\n\t"
+          "ds_read_b128 %2, %4 offset:32\n\t"
+          "ds_read_b128 %3, %4 offset:48\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
+          : "v"(xat)
+          : "memory");
+      if (!any_missing(t, a_lane)) break;
+      if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {  // some workgroup is not running: give up
+        give_up();
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+  };
+
+  // x of (entry, piece hc) from memory into the A registers.  These loads are the youngest of the
+  // wave: everything in its ring lands with them.
+  auto build = [&](const half_t *x, int x_word, int x_src, int k_in, int m_rows, int hc) {
+    const bool active = a_match && a_m < m_rows;
+    const int64_t at = (int64_t)a_m * k_in + hc * 256 + a_off;
+    uint4_t t[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) t[w] = uint4_t{0u, 0u, 0u, 0u};
+    const half_t *p = (x_word >= 0 ? reinterpret_cast<const half_t *>(ex16 + x_word) : x) + at;
+    if (x_word >= 0) wait_own_share(x_src);
+    const unsigned polls_allowed = spin_limit >> 4;
+    unsigned polls = 0;
+    for (;;) {
+      if (active) {
+        asm volatile(
+            "global_load_dwordx4 %0, %4, off sc1\n\t"
+            "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
+            "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
+            "global_load_dwordx4 %3, %4, off offset:48 sc1"
+            : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
+            : "v"(p)
+            : "memory");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
+      if (x_word < 0 || !any_missing(t, active)) break;
+      if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {
+        give_up();
+        break;
+      }
+      __builtin_amdgcn_s_sleep(2);
+    }
+    if (x_word < 0) to_exchange_form(t);
+    finish_build(t);
+  };
+
+  // one unit: ring slot -> registers -> 8 MFMAs -> this lane's group sums into tot.  fresh (batch 1):
+  // the unit brought another piece of x along; it goes into the A registers first, and its sums are
+  // taken while the unit's products run
+  auto consume = [&](int s, float (&tot)[MC], bool fresh, int d, int hc) {
+#if GQ_FLOW_EXP & 1
+    return;
+#endif
+    const uint32_t at = ring_rd + (uint32_t)s * kSlot;
     uint4_t w0, w1;
     uint32_t sc, bi;
-    asm volatile(
-        "ds_read_b128 %0, %4\n\t"
-        "ds_read_b128 %1, %4 offset:1024\n\t"
-        "ds_read_u16 %2, %5 offset:2048\n\t"
-        "ds_read_u16 %3, %5 offset:2176\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(w0), "=&v"(w1), "=&v"(sc), "=&v"(bi)
-        : "v"(at + lane16), "v"(at + sb_read)
-        : "memory");
-    float4_t acc0 = negcorr, acc1 = negcorr;
+    if (XS && fresh) {
+      const uint32_t xat = a_lane ? at + xa_rd : zeros_rd;
+      uint4_t t[4];
+      asm volatile(
+          "ds_read_b128 %4, %10\n\t"
+          "ds_read_b128 %5, %10 offset:16\n\t"
+          "ds_read_b128 %6, %10 offset:32\n\t"
+          "ds_read_b128 %7, %10 offset:48\n\t"
+          "ds_read_b128 %0, %8\n\t"
+          "ds_read_b128 %1, %8 offset:1024\n\t"
+          "ds_read_u16 %2, %9 offset:2048\n\t"
+          "ds_read_u16 %3, %9 offset:2176\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(w0), "=&v"(w1), "=&v"(sc), "=&v"(bi), "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
+          : "v"(at + lane16), "v"(at + sb_read), "v"(xat)
+          : "memory");
+      const bool from_exchange = uni(cache[d].x_word) >= 0;
+      if (from_exchange) {
+        if (any_missing(t, a_lane)) refetch(s, d, hc, xat, t);
+      } else {
+        to_exchange_form(t);
+      }
+      finish_build(t);
+    } else {
+      asm volatile(
+          "ds_read_b128 %0, %4\n\t"
+          "ds_read_b128 %1, %4 offset:1024\n\t"
+          "ds_read_u16 %2, %5 offset:2048\n\t"
+          "ds_read_u16 %3, %5 offset:2176\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(w0), "=&v"(w1), "=&v"(sc), "=&v"(bi)
+          : "v"(at + lane16), "v"(at + sb_read)
+          : "memory");
+    }
+#if GQ_FLOW_EXP & 2
+    tot[0] += __builtin_bit_cast(float, w0[0] ^ w1[1] ^ sc ^ bi);
+    return;
+#endif
+    float4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[w], raw_codes_c(w0[w], kMaskLo, kMaskHi, kMagicLo, kMagicHi), acc0, 0, 0, 0);
@@ -341,7 +452,9 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     const float bias = (float)__builtin_bit_cast(half_t, (unsigned short)bi);
 #pragma unroll
     for (int e = 0; e < MC; ++e) {
-      const float sum = (kc & 2) ? acc1[e] : acc0[e];
+      // (the offsets of the raw codes come out here rather than where the accumulators start, so
+      // that a unit's products do not wait for the sums of a fresh x)
+      const float sum = ((kc & 2) ? acc1[e] : acc0[e]) + negcorr[e];
       tot[e] = __builtin_fmaf(scale, sum, __builtin_fmaf(bias, xsum[e], tot[e]));
     }
   };
@@ -355,7 +468,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     const int n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
     const int active_waves = min(kFlowWaves, pieces);
     const half_t *x = reinterpret_cast<const half_t *>(uni_ptr(cache[d].x));
-    const int x_word = uni(cache[d].x_word), x_src = uni(cache[d].x_src);
+    const int x_word = uni(cache[d].x_word), x_src = uni(cache[d].x_src), x_id = uni(cache[d].x_id);
     for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
       if (n_hc == 0) continue;
       const int nj = min(PR, nrb - pass * PR);
@@ -366,7 +479,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         for (int e = 0; e < MC; ++e) tot[j][e] = 0.f;
       for (int hcp = 0; hcp < n_hc; ++hcp) {
         const int hc = wave + kFlowWaves * hcp;
-        if (!(xa_x == x && xa_word == x_word && xa_src == x_src && xa_k == k_in && xa_m == m_rows && xa_hc == hc)) {
+        if (!XS && !(xa_x == x && xa_word == x_word && xa_src == x_src && xa_k == k_in && xa_m == m_rows && xa_hc == hc)) {
           build(x, x_word, x_src, k_in, m_rows, hc);
           xa_x = x;
           xa_word = x_word;
@@ -378,10 +491,16 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
 #pragma unroll
         for (int j = 0; j < PR; ++j) {
           if (j >= nj) break;
-          // the unit's three loads have landed when at most those of the D - 1 units after it are out
+          // the unit's loads have landed when at most those of the D - 1 units after it are out (a
+          // unit that brings x along has two more: then this waits for more than it needs)
           if (ahead == D) wait_vm<3 * (D - 1)>();
           else wait_vm<0>();
-          consume(slot, tot[j]);
+          const bool fresh = XS && !(GQ_FLOW_EXP & 4) && (x_id != key_id || hc != key_hc);  // (the producer decided the same)
+          if (fresh) {
+            key_id = x_id;
+            key_hc = hc;
+          }
+          consume(slot, tot[j], fresh, d, hc);
           if (prod.d < n_entries) {
             issue(prod, slot);
             advance(prod);
@@ -391,50 +510,67 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           slot = slot + 1 == D ? 0 : slot + 1;
         }
       }
-      // ---- the pass is done for this wave: its sums go to the mailbox; the wave that completes the
-      // set adds the waves' sums up and stores the results
-      const unsigned set = q % S, use = q / S;
-      float out[PR][MC];
-#pragma unroll
-      for (int j = 0; j < PR; ++j)
-#pragma unroll
-        for (int e = 0; e < MC; ++e) {
-          float v = tot[j][e];
-          v += lane_read(v, lane ^ 16);
-          v += lane_read(v, lane ^ 32);
-          out[j][e] = v;
-        }
-      while (lds_load(&ctl->reduced[set]) < use) __builtin_amdgcn_s_sleep(1);  // the set has been emptied
-      float *box = mail + (set * kFlowWaves + wave) * kMail;
-      if (kc == 0) {
-#pragma unroll
+      // ---- the pass is done for this wave: its sums go to the mailbox
+#if GQ_FLOW_EXP & 8
+      {
+        float live = 0.f;
         for (int j = 0; j < PR; ++j)
-          if (j < nj) {
-#pragma unroll
-            for (int e = 0; e < MC; ++e) box[(j * MC + e) * 16 + n] = out[j][e];
-          }
+          for (int e = 0; e < MC; ++e) live += tot[j][e];
+        if (live != 12345.f) continue;
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-      unsigned before = 0;
-      if (lane == 0) before = __hip_atomic_fetch_add(&ctl->deposited[set], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      before = (unsigned)uni((int)before);
-      if (before + 1u != (unsigned)active_waves) continue;
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#endif
+      const unsigned set = q % S, use = q / S;
+      const unsigned emptied = lds_load(&ctl->reduced[set]);
+      // this wave's sums over its four slices: two swaps of half-waves put the sums of row blocks
+      // (0, 1) and (2, 3) side by side, a swap of 16-lane rows finishes both; lane (n, r) then holds
+      // the sum of row block (0, 2, 1, 3)[r] for weight row n
+      // (in assembly: the compiler's builtin for these swaps lost the second result here and added
+      // a register to itself; the wait states are those the compiler puts between a VALU write
+      // and a swap that reads it)
+      float red[MC];
+#pragma unroll
+      for (int e = 0; e < MC; ++e) {
+        float a0 = tot[0][e], a1 = tot[1][e], a2 = tot[2][e], a3 = tot[3][e];
+        asm volatile(
+            "s_nop 1\n\t"
+            "v_permlane32_swap_b32 %0, %1\n\t"
+            "v_permlane32_swap_b32 %2, %3"
+            : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+        float s01 = a0 + a1, s23 = a2 + a3;
+        asm volatile(
+            "s_nop 1\n\t"
+            "v_permlane16_swap_b32 %0, %1"
+            : "+v"(s01), "+v"(s23));
+        red[e] = s01 + s23;
+      }
+      if (emptied < use)
+        while (lds_load(&ctl->reduced[set]) < use) __builtin_amdgcn_s_sleep(1);  // the set has been emptied
+      float *const set_mail = mail + set * kFlowWaves * kMail;  // [e][wave][lane]
+#pragma unroll
+      for (int e = 0; e < MC; ++e) set_mail[(e * kFlowWaves + wave) * 64 + lane] = red[e];
+      // LDS operations of a wave execute in order: the count follows the sums.  (A release fence
+      // would also wait for every load of the ring.)
+      asm volatile("" ::: "memory");
+      if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited[set], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      // the waves take turns at adding the sums up and storing the results
+      if (wave != (int)(q % (unsigned)active_waves)) continue;
+      while (lds_load(&ctl->deposited[set]) < (unsigned)active_waves) __builtin_amdgcn_s_sleep(0);
+      asm volatile("" ::: "memory");
       {
         const int n_out = uni(cache[d].n_out), act = uni(cache[d].act), ex_word = uni(cache[d].ex_word);
         unsigned short *y = reinterpret_cast<unsigned short *>(const_cast<char *>(uni_ptr(cache[d].y)));
         const half_t *out_bias = reinterpret_cast<const half_t *>(uni_ptr(cache[d].out_bias));
-        const float *set_mail = mail + set * kFlowWaves * kMail;
-        for (int t = lane; t < nj * MC * 16; t += 64) {
-          const int n16 = t & 15, m = (t >> 4) % MC, j = t / (16 * MC);
+        const int j = ((kc & 1) << 1) | (kc >> 1);
+        const int row = (b + (pass * PR + j) * G) * 16 + n;
+#pragma unroll
+        for (int e = 0; e < MC; ++e) {
           float sum = 0.f;
-          for (int w = 0; w < active_waves; ++w) sum += set_mail[w * kMail + t];
+          for (int w = 0; w < active_waves; ++w) sum += set_mail[(e * kFlowWaves + w) * 64 + lane];
           sum = -sum;  // (the A registers hold -x)
-          const int row = (b + (pass * PR + j) * G) * 16 + n16;
-          if (m < m_rows && row < n_out) {
+          if (j < nj && e < m_rows && row < n_out) {
             if (out_bias) sum += (float)out_bias[row];
             const unsigned short hv = __builtin_bit_cast(unsigned short, (half_t)apply_activation(sum, act));
-            const int64_t flat = (int64_t)m * n_out + row;
+            const int64_t flat = (int64_t)e * n_out + row;
             __hip_atomic_store(y + flat, hv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (ex_word >= 0) {
               // -y, zero as -0.0; value 8 q + e at place 8 q + (0,2,4,6,1,3,5,7)[e]
@@ -445,12 +581,12 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
             }
           }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // (the mailbox reads are done)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // (the mailbox reads are done)
         if (lane == 0) {
           __hip_atomic_store(&ctl->deposited[set], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          __hip_atomic_store(&ctl->reduced[set], use + 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+          __hip_atomic_store(&ctl->reduced[set], use + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           if ((pass + 1) * PR >= nrb)  // the entry's last pass in this workgroup
-            // (a maximum: the wave that completes the next entry's set may get here first)
+            // (a maximum: the wave that finishes the next entry may get here first)
             __hip_atomic_fetch_max(&ctl->stored, (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
       }

@@ -69,6 +69,7 @@ struct SequencePlan {
   int32_t ex_word[kMaxEntries];  // producer: where the entry's tagged results start in the exchange (-1: none)
   int32_t x_word[kMaxEntries];   // consumer: where its x starts in the exchange (-1: x is read from memory)
   int16_t x_src[kMaxEntries];    // consumer: the entry (of this launch) that produces its x (-1: none)
+  int16_t x_id[kMaxEntries];     // the first entry of the launch that reads the same x (same place, same producer, same shape)
   int16_t need[kMaxEntries];     // entries of this launch that must be reported complete before this one starts
   int32_t uses_exchange;
   int32_t exchange_values;       // results the launch puts into the exchange (a multiple of 64)

@@ -946,6 +946,15 @@ void plan_launch(const gq_gemv_desc *e, int n, int64_t first, bool any_fit, Sequ
     plan.need[i] = 0;
     plan.x_word[i] = plan.ex_word[src] + (int32_t)(((const char *)e[i].x - (const char *)e[src].y) / 2);
   }
+  for (int i = 0; i < n; ++i) {
+    plan.x_id[i] = (int16_t)i;
+    for (int j = 0; j < i; ++j)
+      if (e[j].x == e[i].x && plan.x_word[j] == plan.x_word[i] && plan.x_src[j] == plan.x_src[i] && e[j].k_in == e[i].k_in &&
+          e[j].m_rows == e[i].m_rows) {
+        plan.x_id[i] = (int16_t)j;
+        break;
+      }
+  }
 }
 
 }  // namespace
