@@ -38,26 +38,32 @@ constexpr int kFlowWaves = 16;
 constexpr int kFlowThreads = kFlowWaves * 64;
 constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
 constexpr int kFlowPR = 4;              // row blocks per pass (their running sums stay in registers)
-// At batch 1 a ring slot also has room for the 256 values of x that its unit multiplies (512 bytes):
-// the producer fetches them with the first unit that needs them, ahead of time like the weights,
-// and in the order of the wave's loads they arrive before that unit -- no wait for x drains the ring.
-constexpr bool flow_x_in_slot(int mc) { return mc == 1; }
-constexpr int flow_slot_bytes(int mc) { return kUnitBytes + (flow_x_in_slot(mc) ? 512 : 0); }
+// A ring slot also has room for the 256 values of x that its unit multiplies (512 bytes): the
+// producer fetches them with the first unit that needs them, ahead of time like the weights, and
+// in the order of the wave's loads they arrive before that unit -- no wait for x drains the ring.
+constexpr int flow_slot_bytes(int) { return kUnitBytes + 512; }
 // ring slots per wave and sets of mailboxes, by batch capacity (160 KiB of LDS)
-constexpr int flow_depth(int mc) { return mc == 2 ? 4 : 3; }
-constexpr int flow_sets(int mc) { return mc == 2 ? 1 : 2; }
+constexpr int flow_depth(int) { return 3; }
+constexpr int flow_sets(int) { return 2; }
 
-struct FlowEntry {  // what the work loop needs of an entry, in LDS
+struct FlowEntry {  // what the kernel needs of an entry, in LDS
+  // the 16 bytes the work loop reads per entry, as one LDS read
+  int k_in;
+  int x_word;        // where x starts in the exchange (-1: in memory at x)
+  short nrb, x_src;  // row blocks of this workgroup; producer of x in this launch (-1: none)
+  short x_id;        // the first entry of the launch that reads the same x (same values at the same place)
+  char m_rows, act;
   const char *blob;
   const half_t *x, *out_bias;
   half_t *y;
-  int n_out, k_in;
-  int x_word, ex_word;  // where x starts in the exchange (-1: in memory at x); where the results go (-1: nowhere)
-  short x_src, nrb;     // producer of x in this launch (-1: none); row blocks of this workgroup
-  char m_rows, act;
-  short x_id;           // the first entry of the launch that reads the same x (same values at the same place)
+  int n_out;
+  int ex_word;  // where the results go in the exchange (-1: nowhere)
+  int pad[2];
 };
-static_assert(sizeof(FlowEntry) == 56, "entry cache layout");
+static_assert(sizeof(FlowEntry) == 64 && offsetof(FlowEntry, blob) == 16, "entry cache layout");
+struct FlowHot {  // the first 16 bytes of a FlowEntry, wave-uniform
+  int k_in, x_word, nrb, x_src, x_id, m_rows;
+};
 
 struct FlowControl {
   unsigned deposited[2];  // mailbox deposits into the set since it was last emptied
@@ -77,9 +83,6 @@ constexpr int flow_lds_bytes() {
          flow_sets(MC) * kFlowWaves * kFlowPR * MC * 16 * 4 + (int)sizeof(FlowControl);
 }
 
-#ifndef GQ_FLOW_EXP
-#define GQ_FLOW_EXP 0  // (timing experiments: parts of the kernel switched off)
-#endif
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
 
 // raw_codes() of the other kernel without inline assembly: the compiler's hazard recogniser does
@@ -103,7 +106,6 @@ template <int MC>
 __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int n_entries, int *__restrict__ status,
                                           unsigned *words, unsigned spin_limit, const SequencePlan *plan) {
   constexpr int D = flow_depth(MC), S = flow_sets(MC), PR = kFlowPR;
-  constexpr bool XS = flow_x_in_slot(MC);
   constexpr int kSlot = flow_slot_bytes(MC);
   constexpr int kMail = PR * MC * 16;  // floats a wave deposits per pass: [row block][m][n]
   extern __shared__ __attribute__((aligned(64))) char lds[];
@@ -133,6 +135,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     c.m_rows = (char)e.m_rows;
     c.act = (char)e.activation;
     c.x_id = plan->x_id[i];
+    c.pad[0] = c.pad[1] = 0;
     cache[i] = c;
   }
   if (tid == 0) {
@@ -177,7 +180,21 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   // without data reads zeros
   const uint32_t zeros_rd = (uint32_t)(uintptr_t)ctl->zeros;
   const uint32_t xa_rd = kUnitBytes + (uint32_t)a_off * 2u;
-  const bool a_lane = a_match && a_m == 0;  // (x in the slot is batch 1 only)
+  const bool a_lane = a_match && a_m == 0;  // (batch 1)
+
+  // the hot 16 bytes of entry d as they come out of LDS, and made wave-uniform
+  auto read_hot = [&](int d) { return *reinterpret_cast<const uint4_t *>(&cache[d]); };
+  auto uniform_hot = [&](uint4_t v) {
+    FlowHot h;
+    h.k_in = uni((int)v.x);
+    h.x_word = uni((int)v.y);
+    const int z = uni((int)v.z), w = uni((int)v.w);
+    h.nrb = (short)(z & 0xFFFF);
+    h.x_src = (short)(z >> 16);
+    h.x_id = (short)(w & 0xFFFF);
+    h.m_rows = (signed char)((w >> 16) & 0xFF);
+    return h;
+  };
 
   // ---- the producer: walks this wave's units D ahead of the consumer; all of it wave-uniform
   struct Walk {
@@ -185,15 +202,17 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     int nrb, n_hc, nj, chunks;
     const char *blob;
     // batch 1: the x the A registers would hold at this point of the walk, and where the entry's x is
-    int key_id, key_hc;
+    int key_id, key_hc, x_id;
     const char *xrow;
   };
   auto enter = [&](Walk &w) {  // first unit of entry w.d (n_hc == 0 or nrb == 0: none)
     w.pass = w.hcp = w.j = 0;
     w.nrb = w.n_hc = w.nj = 0;
     if (w.d >= n_entries) return;
-    w.nrb = uni(cache[w.d].nrb);
-    const int k_in = uni(cache[w.d].k_in);
+    const FlowHot h = uniform_hot(read_hot(w.d));
+    w.nrb = h.nrb;
+    w.x_id = h.x_id;
+    const int k_in = h.k_in;
     w.chunks = k_in >> 9;
     const int pieces = k_in >> 8;
     w.n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
@@ -235,15 +254,13 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         : "memory");
   };
   auto issue = [&](Walk &w, int slot) {
-    if (XS) {
-      // the first unit that multiplies another piece of x brings it along: its loads are older than the unit's
-      const int id = uni(cache[w.d].x_id), hc = wave + kFlowWaves * w.hcp;
-      if (id != w.key_id || hc != w.key_hc) {
-        if (id != w.key_id) w.xrow = x_row(w.d);
-        w.key_id = id;
-        w.key_hc = hc;
-        issue_x(w.xrow, hc, slot);
-      }
+    // the first unit that multiplies another piece of x brings it along: its loads are older than the unit's
+    const int id = w.x_id, hc = wave + kFlowWaves * w.hcp;
+    if (id != w.key_id || hc != w.key_hc) {
+      if (id != w.key_id) w.xrow = x_row(w.d);
+      w.key_id = id;
+      w.key_hc = hc;
+      issue_x(w.xrow, hc, slot);
     }
     const int64_t block = (int64_t)(b + (w.pass * PR + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
     const char *src = w.blob + block * (2 * kUnitBytes) + hpar * 2048;
@@ -280,9 +297,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   float4_t negcorr = {0.f, 0.f, 0.f, 0.f}, xsum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int w = 0; w < 4; ++w) xa[w] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-  const half_t *xa_x = nullptr;
-  int xa_word = -2, xa_src = -2, xa_k = 0, xa_m = 0, xa_hc = -1;
-  int key_id = -1, key_hc = -1;  // batch 1
+  int key_id = -1, key_hc = -1;  // the piece of x they hold
 
   auto give_up = [&]() {
     if (lane == 0) {
@@ -334,10 +349,13 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   // batch 1, a unit that brought x along found values that their producer had not delivered when
   // they were fetched: fetch the piece again until it is complete (these loads are the youngest of
   // the wave: everything in its ring lands with them)
-  auto refetch = [&](int s, int d, int hc, uint32_t xat, uint4_t (&t)[4]) {
-    wait_own_share(uni(cache[d].x_src));
+  // The units behind this one in the ring that bring further pieces of the same x along (an entry
+  // with several pieces per wave) fetched theirs at about the same time: they are fetched again with it.
+  auto refetch = [&](int s, int d, int hc, uint32_t xat, uint4_t (&t)[4], int x_src, int step, int more) {
+    wait_own_share(x_src);
     const unsigned polls_allowed = spin_limit >> 4;  // (a poll is a memory round trip)
     unsigned polls = 0;
+    for (int i = 1; i <= more; ++i) issue_x(x_row(d), uni(hc + kFlowWaves * i), uni((s + i * step) % D));
     for (;;) {
       issue_x(x_row(d), hc, s);
       wait_vm<0>();
@@ -359,52 +377,14 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     }
   };
 
-  // x of (entry, piece hc) from memory into the A registers.  These loads are the youngest of the
-  // wave: everything in its ring lands with them.
-  auto build = [&](const half_t *x, int x_word, int x_src, int k_in, int m_rows, int hc) {
-    const bool active = a_match && a_m < m_rows;
-    const int64_t at = (int64_t)a_m * k_in + hc * 256 + a_off;
-    uint4_t t[4];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) t[w] = uint4_t{0u, 0u, 0u, 0u};
-    const half_t *p = (x_word >= 0 ? reinterpret_cast<const half_t *>(ex16 + x_word) : x) + at;
-    if (x_word >= 0) wait_own_share(x_src);
-    const unsigned polls_allowed = spin_limit >> 4;
-    unsigned polls = 0;
-    for (;;) {
-      if (active) {
-        asm volatile(
-            "global_load_dwordx4 %0, %4, off sc1\n\t"
-            "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
-            "global_load_dwordx4 %2, %4, off offset:32 sc1\n\t"
-            "global_load_dwordx4 %3, %4, off offset:48 sc1"
-            : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])
-            : "v"(p)
-            : "memory");
-      }
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3])::"memory");
-      if (x_word < 0 || !any_missing(t, active)) break;
-      if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {
-        give_up();
-        break;
-      }
-      __builtin_amdgcn_s_sleep(2);
-    }
-    if (x_word < 0) to_exchange_form(t);
-    finish_build(t);
-  };
-
   // one unit: ring slot -> registers -> 8 MFMAs -> this lane's group sums into tot.  fresh (batch 1):
   // the unit brought another piece of x along; it goes into the A registers first, and its sums are
   // taken while the unit's products run
-  auto consume = [&](int s, float (&tot)[MC], bool fresh, int d, int hc) {
-#if GQ_FLOW_EXP & 1
-    return;
-#endif
+  auto consume = [&](int s, float (&tot)[MC], bool fresh, int d, int hc, int x_word, int x_src, int step, int more) {
     const uint32_t at = ring_rd + (uint32_t)s * kSlot;
     uint4_t w0, w1;
     uint32_t sc, bi;
-    if (XS && fresh) {
+    if (fresh) {
       const uint32_t xat = a_lane ? at + xa_rd : zeros_rd;
       uint4_t t[4];
       asm volatile(
@@ -420,9 +400,9 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           : "=&v"(w0), "=&v"(w1), "=&v"(sc), "=&v"(bi), "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
           : "v"(at + lane16), "v"(at + sb_read), "v"(xat)
           : "memory");
-      const bool from_exchange = uni(cache[d].x_word) >= 0;
+      const bool from_exchange = x_word >= 0;
       if (from_exchange) {
-        if (any_missing(t, a_lane)) refetch(s, d, hc, xat, t);
+        if (any_missing(t, a_lane)) refetch(s, d, hc, xat, t, x_src, step, more);
       } else {
         to_exchange_form(t);
       }
@@ -438,10 +418,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           : "v"(at + lane16), "v"(at + sb_read)
           : "memory");
     }
-#if GQ_FLOW_EXP & 2
-    tot[0] += __builtin_bit_cast(float, w0[0] ^ w1[1] ^ sc ^ bi);
-    return;
-#endif
     float4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -460,15 +436,18 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   };
 
   // ---- the consumer
+  uint4_t hot_ahead = n_entries > 0 ? read_hot(0) : uint4_t{0u, 0u, 0u, 0u};
   for (int d = 0; d < n_entries; ++d) {
-    const int nrb = uni(cache[d].nrb);
+    // (the next entry's parameters are read from LDS while this one runs: a transition does not wait for them)
+    const FlowHot hot = uniform_hot(hot_ahead);
+    if (d + 1 < n_entries) hot_ahead = read_hot(d + 1);
+    const int nrb = hot.nrb;
     if (nrb == 0) continue;
-    const int k_in = uni(cache[d].k_in), m_rows = uni(cache[d].m_rows);
+    const int k_in = hot.k_in, m_rows = hot.m_rows;
     const int pieces = k_in >> 8;
     const int n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
     const int active_waves = min(kFlowWaves, pieces);
-    const half_t *x = reinterpret_cast<const half_t *>(uni_ptr(cache[d].x));
-    const int x_word = uni(cache[d].x_word), x_src = uni(cache[d].x_src), x_id = uni(cache[d].x_id);
+    const int x_word = hot.x_word, x_src = hot.x_src, x_id = hot.x_id;
     for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
       if (n_hc == 0) continue;
       const int nj = min(PR, nrb - pass * PR);
@@ -479,15 +458,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         for (int e = 0; e < MC; ++e) tot[j][e] = 0.f;
       for (int hcp = 0; hcp < n_hc; ++hcp) {
         const int hc = wave + kFlowWaves * hcp;
-        if (!XS && !(xa_x == x && xa_word == x_word && xa_src == x_src && xa_k == k_in && xa_m == m_rows && xa_hc == hc)) {
-          build(x, x_word, x_src, k_in, m_rows, hc);
-          xa_x = x;
-          xa_word = x_word;
-          xa_src = x_src;
-          xa_k = k_in;
-          xa_m = m_rows;
-          xa_hc = hc;
-        }
 #pragma unroll
         for (int j = 0; j < PR; ++j) {
           if (j >= nj) break;
@@ -495,12 +465,14 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           // unit that brings x along has two more: then this waits for more than it needs)
           if (ahead == D) wait_vm<3 * (D - 1)>();
           else wait_vm<0>();
-          const bool fresh = XS && !(GQ_FLOW_EXP & 4) && (x_id != key_id || hc != key_hc);  // (the producer decided the same)
+          const bool fresh = x_id != key_id || hc != key_hc;  // (the producer decided the same)
           if (fresh) {
             key_id = x_id;
             key_hc = hc;
           }
-          consume(slot, tot[j], fresh, d, hc);
+          // (units of this entry already in the ring that bring the next pieces of x: every nj-th)
+          const int more = fresh ? min((ahead - 1) / nj, n_hc - 1 - hcp) : 0;
+          consume(slot, tot[j], fresh, d, hc, x_word, x_src, nj, more);
           if (prod.d < n_entries) {
             issue(prod, slot);
             advance(prod);
@@ -511,14 +483,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         }
       }
       // ---- the pass is done for this wave: its sums go to the mailbox
-#if GQ_FLOW_EXP & 8
-      {
-        float live = 0.f;
-        for (int j = 0; j < PR; ++j)
-          for (int e = 0; e < MC; ++e) live += tot[j][e];
-        if (live != 12345.f) continue;
-      }
-#endif
       const unsigned set = q % S, use = q / S;
       const unsigned emptied = lds_load(&ctl->reduced[set]);
       // this wave's sums over its four slices: two swaps of half-waves put the sums of row blocks
@@ -551,10 +515,20 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
       // LDS operations of a wave execute in order: the count follows the sums.  (A release fence
       // would also wait for every load of the ring.)
       asm volatile("" ::: "memory");
-      if (lane == 0) __hip_atomic_fetch_add(&ctl->deposited[set], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      // the waves take turns at adding the sums up and storing the results
-      if (wave != (int)(q % (unsigned)active_waves)) continue;
-      while (lds_load(&ctl->deposited[set]) < (unsigned)active_waves) __builtin_amdgcn_s_sleep(0);
+      // the wave that completes the set adds the sums up and stores the results (nobody waits for anybody)
+      unsigned before = 0;
+      if (lane == 0) before = __hip_atomic_fetch_add(&ctl->deposited[set], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      before = (unsigned)uni((int)before);
+      // The arbiter of a SIMD prefers its oldest wave, and an entry is finished when its slowest wave
+      // is: whoever arrives late here gets ahead of the others in the next entry
+      {
+        const unsigned rank = before * 4u / (unsigned)active_waves;
+        if (rank >= 3u) __builtin_amdgcn_s_setprio(3);
+        else if (rank == 2u) __builtin_amdgcn_s_setprio(2);
+        else if (rank == 1u) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+      }
+      if (before + 1u != (unsigned)active_waves) continue;
       asm volatile("" ::: "memory");
       {
         const int n_out = uni(cache[d].n_out), act = uni(cache[d].act), ex_word = uni(cache[d].ex_word);
@@ -618,11 +592,12 @@ __global__ __launch_bounds__(kFlowThreads) void gemv_flow_kernel(const void *ent
   flow_body<MC>(reinterpret_cast<const Entry *>(entries), n_entries, status, words, spin_limit, &plan);
 }
 
-// Can this launch run on the data-flow kernel?  Every weight in the streaming layout, at most four
-// batch rows, and no entry that has to wait for reported completion.
+// Can this launch run on the data-flow kernel?  Every weight in the streaming layout, one batch
+// row (measured at batch 4: the LDS-ring kernel is faster there), and no entry that has to wait
+// for reported completion.
 bool flow_eligible(const gq_gemv_desc *e, int n, const SequencePlan &plan) {
   for (int i = 0; i < n; ++i)
-    if (e[i].scale != nullptr || e[i].bias != nullptr || e[i].m_rows > 4 || plan.need[i] != 0 || e[i].k_in % 512 != 0) return false;
+    if (e[i].scale != nullptr || e[i].bias != nullptr || e[i].m_rows != 1 || plan.need[i] != 0 || e[i].k_in % 512 != 0) return false;
   return true;
 }
 
@@ -630,8 +605,7 @@ int launch_flow(const gq_gemv_desc *host, const gq_gemv_desc *device, int n, int
                 const SequencePlan &plan, int grid, int dev, hipStream_t stream) {
   constexpr int kMaxDevices = 64;
   if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
-  int max_m = 1;
-  for (int i = 0; i < n; ++i) max_m = host[i].m_rows > max_m ? host[i].m_rows : max_m;
+  (void)host;
 #define GQ_FLOW(MC)                                                                                           \
   do {                                                                                                        \
     constexpr int lds_bytes = flow_lds_bytes<MC>();                                                           \
@@ -645,9 +619,7 @@ int launch_flow(const gq_gemv_desc *host, const gq_gemv_desc *device, int n, int
     }                                                                                                         \
     gemv_flow_kernel<MC><<<dim3(grid), dim3(kFlowThreads), lds_bytes, stream>>>(device, n, status, words, spins, plan); \
   } while (0)
-  if (max_m == 1) GQ_FLOW(1);
-  else if (max_m == 2) GQ_FLOW(2);
-  else GQ_FLOW(4);
+  GQ_FLOW(1);
 #undef GQ_FLOW
   return GQ_OK;
 }
