@@ -201,9 +201,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     int d, pass, hcp, j;  // entry, pass of row blocks, this wave's how-manieth 256-feature piece, row block in pass
     int nrb, n_hc, nj, chunks;
     const char *blob;
-    // batch 1: the x the A registers would hold at this point of the walk, and where the entry's x is
-    int key_id, key_hc, x_id;
-    const char *xrow;
   };
   auto enter = [&](Walk &w) {  // first unit of entry w.d (n_hc == 0 or nrb == 0: none)
     w.pass = w.hcp = w.j = 0;
@@ -211,7 +208,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     if (w.d >= n_entries) return;
     const FlowHot h = uniform_hot(read_hot(w.d));
     w.nrb = h.nrb;
-    w.x_id = h.x_id;
     const int k_in = h.k_in;
     w.chunks = k_in >> 9;
     const int pieces = k_in >> 8;
@@ -253,15 +249,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         : "s"(dst), "v"(lane4), "s"(src)
         : "memory");
   };
-  auto issue = [&](Walk &w, int slot) {
-    // the first unit that multiplies another piece of x brings it along: its loads are older than the unit's
-    const int id = w.x_id, hc = wave + kFlowWaves * w.hcp;
-    if (id != w.key_id || hc != w.key_hc) {
-      if (id != w.key_id) w.xrow = x_row(w.d);
-      w.key_id = id;
-      w.key_hc = hc;
-      issue_x(w.xrow, hc, slot);
-    }
+  auto issue = [&](const Walk &w, int slot) {
     const int64_t block = (int64_t)(b + (w.pass * PR + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
     const char *src = w.blob + block * (2 * kUnitBytes) + hpar * 2048;
     const uint32_t dst = ring_rd + (uint32_t)slot * kSlot;
@@ -280,8 +268,6 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   prod.d = -1;
   prod.blob = nullptr;
   prod.chunks = 0;
-  prod.key_id = prod.key_hc = -1;
-  prod.xrow = nullptr;
   next_entry(prod);
   int ahead = 0;  // units issued and not yet consumed
   while (ahead < D && prod.d < n_entries) {
@@ -298,6 +284,8 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
 #pragma unroll
   for (int w = 0; w < 4; ++w) xa[w] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
   int key_id = -1, key_hc = -1;  // the piece of x they hold
+  bool x_requested = false;      // the x of the next unit is on its way into that unit's slot
+  int g1 = 3, g2 = 3;            // loads in the groups issued with the unit before the last, and with the last
 
   auto give_up = [&]() {
     if (lane == 0) {
@@ -351,11 +339,10 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   // the wave: everything in its ring lands with them)
   // The units behind this one in the ring that bring further pieces of the same x along (an entry
   // with several pieces per wave) fetched theirs at about the same time: they are fetched again with it.
-  auto refetch = [&](int s, int d, int hc, uint32_t xat, uint4_t (&t)[4], int x_src, int step, int more) {
-    wait_own_share(x_src);
+  auto refetch = [&](int s, int d, int hc, uint32_t xat, uint4_t (&t)[4], int x_src) {
+    if (x_src >= 0) wait_own_share(x_src);
     const unsigned polls_allowed = spin_limit >> 4;  // (a poll is a memory round trip)
     unsigned polls = 0;
-    for (int i = 1; i <= more; ++i) issue_x(x_row(d), uni(hc + kFlowWaves * i), uni((s + i * step) % D));
     for (;;) {
       issue_x(x_row(d), hc, s);
       wait_vm<0>();
@@ -368,7 +355,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           : "=&v"(t[0]), "=&v"(t[1]), "=&v"(t[2]), "=&v"(t[3])
           : "v"(xat)
           : "memory");
-      if (!any_missing(t, a_lane)) break;
+      if (x_src < 0 || !any_missing(t, a_lane)) break;
       if (polls++ >= polls_allowed || lds_load(&ctl->failed)) {  // some workgroup is not running: give up
         give_up();
         break;
@@ -380,7 +367,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   // one unit: ring slot -> registers -> 8 MFMAs -> this lane's group sums into tot.  fresh (batch 1):
   // the unit brought another piece of x along; it goes into the A registers first, and its sums are
   // taken while the unit's products run
-  auto consume = [&](int s, float (&tot)[MC], bool fresh, int d, int hc, int x_word, int x_src, int step, int more) {
+  auto consume = [&](int s, float (&tot)[MC], bool fresh, bool requested, int d, int hc, int x_word, int x_src) {
     const uint32_t at = ring_rd + (uint32_t)s * kSlot;
     uint4_t w0, w1;
     uint32_t sc, bi;
@@ -401,11 +388,9 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           : "v"(at + lane16), "v"(at + sb_read), "v"(xat)
           : "memory");
       const bool from_exchange = x_word >= 0;
-      if (from_exchange) {
-        if (any_missing(t, a_lane)) refetch(s, d, hc, xat, t, x_src, step, more);
-      } else {
-        to_exchange_form(t);
-      }
+      // (not requested: the first unit of the launch, or an entry after one without work for this wave)
+      if (!requested || (from_exchange && any_missing(t, a_lane))) refetch(s, d, hc, xat, t, from_exchange ? x_src : -1);
+      if (!from_exchange) to_exchange_form(t);
       finish_build(t);
     } else {
       asm volatile(
@@ -448,6 +433,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     const int n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
     const int active_waves = min(kFlowWaves, pieces);
     const int x_word = hot.x_word, x_src = hot.x_src, x_id = hot.x_id;
+    const char *const xrow = x_word >= 0 ? reinterpret_cast<const char *>(ex16 + x_word) : uni_ptr(cache[d].x);
     for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
       if (n_hc == 0) continue;
       const int nj = min(PR, nrb - pass * PR);
@@ -461,25 +447,61 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
 #pragma unroll
         for (int j = 0; j < PR; ++j) {
           if (j >= nj) break;
-          // the unit's loads have landed when at most those of the D - 1 units after it are out (a
-          // unit that brings x along has two more: then this waits for more than it needs)
-          if (ahead == D) wait_vm<3 * (D - 1)>();
-          else wait_vm<0>();
-          const bool fresh = x_id != key_id || hc != key_hc;  // (the producer decided the same)
+          const bool fresh = x_id != key_id || hc != key_hc;
+          const bool requested = fresh && x_requested;
           if (fresh) {
             key_id = x_id;
             key_hc = hc;
           }
-          // (units of this entry already in the ring that bring the next pieces of x: every nj-th)
-          const int more = fresh ? min((ahead - 1) / nj, n_hc - 1 - hcp) : 0;
-          consume(slot, tot[j], fresh, d, hc, x_word, x_src, nj, more);
+          // Loads of a wave land in the order issued.  After this unit's three came the groups issued
+          // with the two units before it (three loads each, two more with a request for x); a
+          // requested x came just before the last of those groups.
+          if (ahead < D || (requested && g2 == 2)) {
+            wait_vm<0>();
+          } else if (requested) {
+            wait_vm<3>();
+          } else {
+            const int after = g1 + g2;
+            if (after == 6) wait_vm<6>();
+            else if (after == 8) wait_vm<8>();
+            else wait_vm<10>();
+          }
+          consume(slot, tot[j], fresh, requested, d, hc, x_word, x_src);
+          // ---- what this wave multiplies next: another piece of x is requested now, one unit ahead.
+          // (Further ahead, results of an entry just before are not there yet, and what a request
+          // brings instead has to be fetched again with every load of the ring in front of it.)
+          int nx_hc = -1, nx_id = x_id;  // nx_hc < 0: the same piece, or nothing known
+          const char *nx_row = xrow;
+          if (j + 1 < nj) {
+          } else if (hcp + 1 < n_hc) {
+            nx_hc = hc + kFlowWaves;
+          } else if ((pass + 1) * PR < nrb) {
+            if (n_hc > 1) nx_hc = wave;
+          } else if (d + 1 < n_entries) {
+            const FlowHot next = uniform_hot(hot_ahead);
+            if (next.nrb > 0 && wave < (next.k_in >> 8)) {
+              nx_hc = wave;
+              nx_id = next.x_id;
+              if (nx_id != x_id)
+                nx_row = next.x_word >= 0 ? reinterpret_cast<const char *>(ex16 + next.x_word) : uni_ptr(cache[d + 1].x);
+            }
+          }
+          const int next_slot = slot + 1 == D ? 0 : slot + 1;
+          x_requested = nx_hc >= 0 && (nx_id != key_id || nx_hc != key_hc);
+          g1 = g2;
+          g2 = 0;
+          if (x_requested) {
+            issue_x(nx_row, nx_hc, next_slot);
+            g2 = 2;
+          }
           if (prod.d < n_entries) {
             issue(prod, slot);
             advance(prod);
+            g2 += 3;
           } else {
             --ahead;
           }
-          slot = slot + 1 == D ? 0 : slot + 1;
+          slot = next_slot;
         }
       }
       // ---- the pass is done for this wave: its sums go to the mailbox
