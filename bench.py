@@ -264,6 +264,9 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     return r
 
 
+FLOW_KERNEL_MODES = ("sequence_decoder_data_flow_streaming_layout", "sequence_no_waits_streaming_layout")
+
+
 def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384, modes=None):
     """Benchmark configuration 5: 28 layers x {4 x [4096x4096], [16384x4096], [4096x16384]} as a
     sequence of fused GEMVs, every matrix distinct (3.17 GB of packed weight in total)."""
@@ -419,7 +422,10 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                          "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
                          "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0),
-                         "roofline": hbm_roofline("gemv_stream_kernel", w_bytes, ms)}
+                         # batch 1, every weight in the streaming layout, every dependency carried by data: the
+                         # data-flow kernel; anything else: the LDS-ring kernel
+                         "roofline": hbm_roofline("gemv_flow_kernel" if m_rows == 1 and mode in FLOW_KERNEL_MODES else "gemv_stream_kernel",
+                                                  w_bytes, ms)}
         # the timed passes computed something: what the buffers hold now (the last layer's outputs)
         # equals single-call GEMVs on the same weights and the inputs the device had
         worst = 0.0
@@ -449,6 +455,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", default="all", choices=["decompress", "compress", "gemv", "kn", "gemm", "stack", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--stack-modes", default="",
+                    help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
+    ap.add_argument("--stack-batches", default="1,4", help="batch sizes of the stack runs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB device copy (known traffic) for scaling profiler byte counters")
     args = ap.parse_args()
@@ -554,15 +563,14 @@ def main():
             torch.cuda.empty_cache()
     if args.only in ("stack", "all"):
         extra["stack"] = []
-        for m in (1, 4):
-            r = bench_stack(hip, device, m, passes=20, warmup=3)
+        modes = tuple(m for m in args.stack_modes.split(",") if m) or None
+        for m in (int(v) for v in args.stack_batches.split(",")):
+            r = bench_stack(hip, device, m, passes=20, warmup=3, modes=modes)
             extra["stack"].append(r)
-            for mode in ("per_launch_graph", "sequence_sequential_block", "sequence_parallel_block",
-                         "sequence_parallel_block_fused_qkv", "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout",
-                         "sequence_decoder_data_flow", "sequence_decoder_data_flow_streaming_layout",
-                         "sequence_no_waits", "sequence_no_waits_streaming_layout"):
-                log(f"  stack m={m} {mode}: {r[mode]['us_per_pass']:.0f} us/pass, {r[mode]['weight_gbs']:.0f} GB/s weights "
-                    f"({r[mode]['hbm_frac']:.1%})")
+            for mode, v in r.items():
+                if isinstance(v, dict) and "us_per_pass" in v:
+                    log(f"  stack m={m} {mode}: {v['us_per_pass']:.0f} us/pass, {v['weight_gbs']:.0f} GB/s weights "
+                        f"({v['hbm_frac']:.1%}) [{v['roofline']['kernel']}]")
             torch.cuda.empty_cache()
     extra["bench_wall_s"] = round(time.time() - t_begin, 1)
 
