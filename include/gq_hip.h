@@ -182,7 +182,11 @@ int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16
  *
  * For group_size 64, k_in % 512 == 0, m_rows <= 4 and 16-byte aligned pointers the whole sequence
  * runs as one persistent kernel (one workgroup per compute unit) that streams the packed weights
- * without a gap between entries; any other sequence runs as one launch per entry.
+ * without a gap between entries; any other sequence runs as one launch per entry.  There are two
+ * such kernels: launches of one batch row whose weights are all in the streaming layout (below) and
+ * whose entries need nothing but the results they read as x run on the faster of the two; every
+ * other launch runs on the general one.  The choice is made per launch of up to 128 entries and
+ * changes no result beyond the tolerance of the fused paths.
  *
  *   descs         host copy of the entries (validated here, not read after the call returns)
  *   descs_device  device copy of the same `count` entries (read by the kernel)
@@ -197,9 +201,12 @@ int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16
  * gq_gemv_sequence_f16     keeps the per-workgroup progress words in a block that the library
  *                          holds per device: at most ONE sequence may run on a device at a time.
  * gq_gemv_sequence_ws_f16  takes them from `workspace` (device memory, 256-byte aligned,
- *                          gq_gemv_sequence_workspace_bytes() bytes, zeroed by the caller once; the
- *                          kernel leaves it zeroed), so that the library holds no state for the
- *                          call: sequences with workspaces of their own may be enqueued on
+ *                          gq_gemv_sequence_workspace_bytes() bytes -- progress words and the
+ *                          buffers through which results travel from entry to entry inside a
+ *                          launch -- zeroed by the caller once, before its first use; after that
+ *                          the calls that use it keep it in the state the next one expects), so
+ *                          that the library holds no state for the call: sequences with
+ *                          workspaces of their own may be enqueued on
  *                          different streams and captured in different graphs, as long as the
  *                          caller orders them (events) so that two persistent kernels never run at
  *                          the same time -- each needs every compute unit.  spin_limit <= 0 selects
