@@ -8,8 +8,8 @@
 //   word  = c0 << 12 | c1 << 8 | c2 << 4 | c3               (:193-195)
 // Every fp16 operation is rounded on its own: sums/differences are native fp16 ops, quotients
 // are correctly rounded fp32 divisions rounded again to fp16 (24 >= 2*11+2 bits makes the double
-// rounding exact).  Compiled with -ffp-contract=off.  HBM-bound: 2 B read, 0.5 + 4/gs B written
-// per element.
+// rounding exact), or products with a correctly rounded reciprocal where that is proved equal.
+// Compiled with -ffp-contract=off.  HBM-bound: 2 B read, 0.5 + 4/gs B written per element.
 #include "gq_common.h"
 
 namespace gq {
@@ -19,22 +19,22 @@ constexpr int kThreads = 256;
 
 __device__ __forceinline__ bool nonfinite_bits(uint32_t h) { return (h & 0x7c00u) == 0x7c00u; }
 
-// f16(diff / scale), correctly rounded, from a reciprocal shared by the group: one Newton step on
-// the fp32 product.  Why that is enough: the residual e = diff - scale * t is exact (an fma of
-// 11-bit by 24-bit operands whose result cancels down to a few bits), so t2 = t + e * r lies
-// within one fp32 ulp of the true quotient, while a quotient of two 11-bit significands is at
-// least 2^-22 (relative, in [1, 2)) away from every fp16 rounding boundary -- four fp32 ulps.  No
-// boundary can lie between t2 and the quotient, so rounding t2 rounds the quotient.
-__device__ __forceinline__ half_t divide(half_t diff, float scale_f32, float recip) {
-  const float d = (float)diff;
-  const float t = __builtin_fmaf(d, recip, 0.f);  // the product, as a mixed-precision fma that reads diff as fp16
-  const float e = __builtin_fmaf(-scale_f32, t, d);
-  return (half_t)__builtin_fmaf(e, recip, t);
+// f16(diff / scale) from the reciprocal of the scale, shared by the group: ONE fp32 product, rounded
+// again to fp16.  Why that is enough: the reciprocal is the correctly rounded one (an IEEE division,
+// once per group), so the product lies within 1.5 fp32 ulps of the true quotient (half an ulp of the
+// reciprocal, scaled by a quotient below 2, and half an ulp of the product), while a quotient of two
+// 11-bit significands D/S in [1, 2) is at least 1/(S 2^11) > 2^-22 -- two fp32 ulps -- away from
+// every fp16 rounding boundary M/2^11, M odd (|D 2^11 - M S| is a nonzero integer).  No boundary
+// can lie between the product and the quotient, so rounding the product rounds the quotient.  (Where
+// the quotient is subnormal in fp16 the boundaries are closer; every such quotient gives code 0.)
+__device__ __forceinline__ half_t divide(half_t diff, float recip) {
+  // the product as a mixed-precision fma that reads diff as fp16 and writes fp16
+  return (half_t)__builtin_fmaf((float)diff, recip, 0.f);
 }
 
-__device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float scale_f32, float recip) {
+__device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float recip) {
   const half_t diff = v - lo;
-  const half_t quot = divide(diff, scale_f32, recip);
+  const half_t quot = divide(diff, recip);
   int c = (int)__builtin_rintf((float)quot);
   c = c < 0 ? 0 : (c > 15 ? 15 : c);  // no effect wherever the reference is well defined
   return (uint32_t)c;
@@ -42,8 +42,10 @@ __device__ __forceinline__ uint32_t quantize(half_t v, half_t lo, float scale_f3
 
 // LANES lanes share one group; each lane holds 8 (or 16) consecutive elements (one or two 16-byte
 // loads) and writes the uint16 words made from them as one 32-bit (64-bit) store.
-// The kernel is bound by instruction issue, not by HBM, so the work is done two elements per
-// instruction wherever a packed fp16 form exists (the roundings are those of the scalar forms).
+// The work is done two elements per instruction wherever a packed fp16 form exists (the roundings
+// are those of the scalar forms).  What bounds the kernel is neither that arithmetic (a third fewer
+// instructions changed nothing) nor the loads in flight (more of them per thread made it slower):
+// without its stores of packed words the same kernel runs at 93 % of the HBM peak, with them at 69 %.
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
 
 // packed minimum / maximum as single instructions (the generic builtins first quieten their
@@ -63,23 +65,19 @@ __device__ __forceinline__ half2_t pk_max(half2_t a, half2_t b) {
 // 16 LANES -- half the lanes per group: one shuffle round less, and the scale, reciprocal and
 // store of the group's statistics amortised over twice the elements)
 template <int LANES, int V>
-__global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__restrict__ t, uint32_t *__restrict__ packed,
-                                                            half_t *__restrict__ scale, half_t *__restrict__ bias,
-                                                            int32_t *__restrict__ flag, int64_t n_items) {
-  const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  const bool live = item < n_items;
+__device__ __forceinline__ void compress_item(const uint4_t (&q)[V], int64_t item, bool live, uint32_t *__restrict__ packed,
+                                              half_t *__restrict__ scale, half_t *__restrict__ bias,
+                                              int32_t *__restrict__ flag) {
   half2_t h[4 * V];
-  ushort2_t exponents = {0, 0};  // maximum of the exponent fields: 0x7c00 = Inf or NaN seen
+  half2_t poison = {(half_t)0.f, (half_t)0.f};  // sum of 0 * x: NaN once an Inf or NaN has been seen
+  const half2_t zero_pair = {(half_t)0.f, (half_t)0.f};
 #pragma unroll
   for (int v = 0; v < V; ++v) {
-    uint4_t q = {0u, 0u, 0u, 0u};
-    if (live) q = __builtin_nontemporal_load(t + item * V + v);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const uint32_t w = q[d];  // (a bit cast straight from a vector element reads element 0)
+      const uint32_t w = q[v][d];  // (a bit cast straight from a vector element reads element 0)
       h[4 * v + d] = __builtin_bit_cast(half2_t, w);
-      const uint32_t e = w & 0x7c007c00u;
-      exponents = __builtin_elementwise_max(exponents, __builtin_bit_cast(ushort2_t, e));
+      poison = __builtin_elementwise_fma(h[4 * v + d], zero_pair, poison);
     }
   }
   half2_t mx = pk_max(pk_max(h[0], h[1]), pk_max(h[2], h[3]));
@@ -103,38 +101,78 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__res
   // scale 0 (a constant group, or a range too small for fp16): every code is 0; dividing by 1 gives
   // that without a branch, because every difference is then below 2^-20
   const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
-  const float recip = __builtin_amdgcn_rcpf(sc32);
+  const float recip = 1.0f / sc32;  // (correctly rounded: the compiler's IEEE division)
   const half2_t lo_pair = {lo, lo}, ceiling = {(half_t)1039.0f, (half_t)1039.0f}, magic = {(half_t)1024.0f, (half_t)1024.0f};
-  uint32_t m[4 * V];  // codes of elements (2d, 2d + 1) at bits 3:0 and 19:16
+  // Each step for all pairs before the next step for any: an instruction that reads what the one
+  // before it wrote with a half-word selection costs a wait state on this hardware, and the
+  // compiler's own order (one pair at a time) put one in front of three instructions in five.
+  half2_t diff[4 * V], quot[4 * V];
 #pragma unroll
-  for (int d = 0; d < 4 * V; ++d) {
-    const half2_t diff = h[d] - lo_pair;
-    const half2_t quot = {divide(diff[0], sc32, recip), divide(diff[1], sc32, recip)};
-    // quot + 1024 rounds to an integer, ties to even (the ulp of fp16 at 1024 is 1): that is
-    // 1024 + rint(quot), with the code in the low mantissa bits.  Codes above 15 are clipped (no
-    // effect wherever the reference is well defined).
-    const half2_t biased = pk_min(quot + magic, ceiling);
-    m[d] = __builtin_bit_cast(uint32_t, biased) & 0x000F000Fu;
-  }
+  for (int d = 0; d < 4 * V; ++d) diff[d] = h[d] - lo_pair;
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int d = 0; d < 4 * V; ++d) quot[d][0] = divide(diff[d][0], recip);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int d = 0; d < 4 * V; ++d) quot[d][1] = divide(diff[d][1], recip);
+  __builtin_amdgcn_sched_barrier(0);
+  // quot + 1024 rounds to an integer, ties to even (the ulp of fp16 at 1024 is 1): that is
+  // 1024 + rint(quot) = 0x6400 + code as a bit pattern.  Codes above 15 are clipped (no effect
+  // wherever the reference is well defined; a NaN becomes 15).
+#pragma unroll
+  for (int d = 0; d < 4 * V; ++d) quot[d] = quot[d] + magic;
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int d = 0; d < 4 * V; ++d) quot[d] = pk_min(quot[d], ceiling);
+  // A uint16 word is 4096 c0 + 256 c1 + 16 c2 + c3: two dot products of 16-bit pairs, the second
+  // starting from the first; the 0x6400 of the four patterns is taken out where the sum starts
+  // (modulo 2^32, and the result is below 2^16).
+  const ushort2_t hi_weights = {4096, 256}, lo_weights = {16, 1};
+  const uint32_t start = 0u - 0x6400u * (4096u + 256u + 16u + 1u);
   uint32_t word[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) {
-    const uint32_t w0 = ((m[4 * v] << 12) | (m[4 * v] >> 8) | (m[4 * v + 1] << 4) | (m[4 * v + 1] >> 16)) & 0xFFFFu;
-    const uint32_t w1 = ((m[4 * v + 2] << 12) | (m[4 * v + 2] >> 8) | (m[4 * v + 3] << 4) | (m[4 * v + 3] >> 16)) & 0xFFFFu;
-    word[v] = w0 | (w1 << 16);
+    uint32_t w16[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t part = __builtin_amdgcn_udot2(__builtin_bit_cast(ushort2_t, quot[4 * v + 2 * i + 1]), lo_weights, start, false);
+      w16[i] = __builtin_amdgcn_udot2(__builtin_bit_cast(ushort2_t, quot[4 * v + 2 * i]), hi_weights, part, false);
+    }
+    word[v] = __builtin_amdgcn_perm(w16[1], w16[0], 0x05040100u);  // the low halves of both, side by side
   }
   if (live) {
+    // (streaming stores: nothing reads the result soon; 0.4 us of 31 on 4096 x 16384)
     if (V == 1) {
-      packed[item] = word[0];
+      __builtin_nontemporal_store(word[0], packed + item);
     } else {
-      *reinterpret_cast<uint2_t *>(packed + item * 2) = uint2_t{word[0], word[V - 1]};
+      __builtin_nontemporal_store(uint2_t{word[0], word[V - 1]}, reinterpret_cast<uint2_t *>(packed + item * 2));
     }
-    if ((item & (LANES - 1)) == 0) {
-      scale[item / LANES] = sc;
-      bias[item / LANES] = lo;
-    }
-    if (flag && (exponents[0] == 0x7c00 || exponents[1] == 0x7c00)) *flag = 1;
+    if (flag && (poison[0] != poison[0] || poison[1] != poison[1])) *flag = 1;
   }
+  // (Collecting the statistics of four groups in one lane for 8-byte stores was measured: the
+  // shuffles cost what the wider stores save.)
+  if (live && (item & (LANES - 1)) == 0) {
+    scale[item / LANES] = sc;
+    bias[item / LANES] = lo;
+  }
+}
+
+template <int LANES, int V>
+__global__ __launch_bounds__(kThreads) void compress_kernel(const uint4_t *__restrict__ t, uint32_t *__restrict__ packed,
+                                                            half_t *__restrict__ scale, half_t *__restrict__ bias,
+                                                            int32_t *__restrict__ flag, int64_t n_items) {
+  // One item per thread and as many workgroups as that takes.  (Measured on 4096 x 16384: several
+  // items per thread with all their loads issued first, 34 to 38 us, and a fixed grid of 1024 to
+  // 8192 workgroups that loads an item ahead, 34 to 37 us, against 31 us.)
+  const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const bool live = item < n_items;
+  uint4_t q[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    q[v] = uint4_t{0u, 0u, 0u, 0u};
+    if (live) q[v] = __builtin_nontemporal_load(t + item * V + v);
+  }
+  compress_item<LANES, V>(q, item, live, packed, scale, bias, flag);
 }
 
 // Any group_size % 4 == 0: one lane per group.
@@ -159,10 +197,10 @@ __global__ __launch_bounds__(kThreads) void compress_generic_kernel(const half_t
   scale[g] = sc;
   bias[g] = lo;
   const float sc32 = (float)sc == 0.f ? 1.0f : (float)sc;
-  const float recip = __builtin_amdgcn_rcpf(sc32);
+  const float recip = 1.0f / sc32;  // (correctly rounded: the compiler's IEEE division)
   for (int i = 0; i < group_size / 4; ++i) {
     uint32_t w = 0;
-    for (int j = 0; j < 4; ++j) w = (w << 4) | quantize(src[4 * i + j], lo, sc32, recip);
+    for (int j = 0; j < 4; ++j) w = (w << 4) | quantize(src[4 * i + j], lo, recip);
     packed[g * (group_size / 4) + i] = (uint16_t)w;
   }
   if (bad && flag) *flag = 1;

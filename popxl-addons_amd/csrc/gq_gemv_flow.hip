@@ -34,6 +34,10 @@
 namespace gq {
 namespace {
 
+// cache policy of the weight loads (every byte is read once per launch)
+#ifndef GQ_FLOW_WEIGHT_POLICY
+#define GQ_FLOW_WEIGHT_POLICY " nt"
+#endif
 constexpr int kFlowWaves = 16;
 constexpr int kFlowThreads = kFlowWaves * 64;
 constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
@@ -256,9 +260,9 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
         "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %1, %3\n\t"
-        "global_load_lds_dwordx4 %1, %3 offset:1024\n\t"
-        "global_load_lds_dword %2, %3 offset:2048"
+        "global_load_lds_dwordx4 %1, %3" GQ_FLOW_WEIGHT_POLICY "\n\t"
+        "global_load_lds_dwordx4 %1, %3 offset:1024" GQ_FLOW_WEIGHT_POLICY "\n\t"
+        "global_load_lds_dword %2, %3 offset:2048" GQ_FLOW_WEIGHT_POLICY
         :
         : "s"(dst), "v"(lane16), "v"(sb_fetch), "s"(src)
         : "memory");
