@@ -1,13 +1,15 @@
 // The data-flow kernel of the GEMV sequence: a persistent kernel for launches whose weights are in
 // the streaming layout and whose dependencies all travel through the exchange (a decoder's layer
-// stack at batch 1 to 4).  The LDS-ring kernel of gq_gemv_stream.hip serves everything else.
+// stack at batch 1; the arithmetic is laid out for up to four batch rows, but measured at batch 4
+// the LDS-ring kernel is faster, so only one row is instantiated).  The LDS-ring kernel of
+// gq_gemv_stream.hip serves everything else.
 //
 // Why a second kernel: a stack of dependent GEMVs stalls at every layer boundary (the next layer
 // needs every output of this one), and a stall only costs nothing if the weights keep streaming
 // into a buffer meanwhile AND the arithmetic then catches up faster than memory delivers.  This
 // kernel is built for few instructions per byte: 16 waves per compute unit (four per SIMD), a work
 // unit of 16 weight rows x 256 input features (2304 bytes: three direct-to-LDS loads into a
-// four-deep ring per wave, 144 KiB per compute unit in flight or buffered, issued across entry
+// three-slot ring per wave, 110 KiB per compute unit in flight or buffered, issued across entry
 // boundaries -- weights never depend on results), and no staging of x at all.
 //
 // Arithmetic (v_mfma_f32_16x16x32_f16, one per 512 weights).  B operand = raw codes: the nibble
@@ -34,17 +36,16 @@
 namespace gq {
 namespace {
 
-// cache policy of the weight loads (every byte is read once per launch)
-#ifndef GQ_FLOW_WEIGHT_POLICY
+// cache policy of the weight loads: every byte is read once per launch (0.5 to 1.5 % of a pass
+// against the default policy)
 #define GQ_FLOW_WEIGHT_POLICY " nt"
-#endif
 constexpr int kFlowWaves = 16;
 constexpr int kFlowThreads = kFlowWaves * 64;
 constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
 constexpr int kFlowPR = 4;              // row blocks per pass (their running sums stay in registers)
-// A ring slot also has room for the 256 values of x that its unit multiplies (512 bytes): the
-// producer fetches them with the first unit that needs them, ahead of time like the weights, and
-// in the order of the wave's loads they arrive before that unit -- no wait for x drains the ring.
+// A ring slot also has room for the 256 values of x that its unit multiplies (512 bytes): they are
+// requested one unit ahead, in front of the weight loads issued at the same time, and in the order
+// of the wave's loads they arrive before that unit -- no wait for x drains the ring.
 constexpr int flow_slot_bytes(int) { return kUnitBytes + 512; }
 // ring slots per wave and sets of mailboxes, by batch capacity (160 KiB of LDS)
 constexpr int flow_depth(int) { return 3; }
