@@ -565,7 +565,9 @@ def main():
         extra["stack"] = []
         modes = tuple(m for m in args.stack_modes.split(",") if m) or None
         for m in (int(v) for v in args.stack_batches.split(",")):
-            r = bench_stack(hip, device, m, passes=20, warmup=3, modes=modes)
+            # (a pass takes 0.5 to 1.6 ms; the first few dozen launches after a pause run up to 15 % slower
+            # than the steady state, so they are warm-up)
+            r = bench_stack(hip, device, m, passes=100, warmup=40, modes=modes)
             extra["stack"].append(r)
             for mode, v in r.items():
                 if isinstance(v, dict) and "us_per_pass" in v:
