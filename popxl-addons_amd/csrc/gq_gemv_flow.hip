@@ -42,7 +42,16 @@ namespace {
 constexpr int kFlowWaves = 16;
 constexpr int kFlowThreads = kFlowWaves * 64;
 constexpr int kUnitBytes = 2048 + 256;  // two 1 KiB loads of packed words; 32 words of scales, 32 of biases
-constexpr int kFlowPR = 4;              // row blocks per pass (their running sums stay in registers)
+constexpr int kFlowPR = 4;              // row blocks per pass at most (their running sums stay in registers)
+// An entry whose results a later entry of the launch reads, and that has kEarlyMinBlocks row blocks
+// or more in a workgroup, passes them on kEarlyRows row blocks at a time (a reduction each) instead
+// of all at the end.  The reader's first pieces are the producer's first row blocks: they are then
+// on their way while the rest of the producer still streams, and the reader's waves do not
+// meet a wait that sends them on at different times.  Measured on the 6B decoder stack (up feeds
+// down, four row blocks a workgroup): 693 -> 627 us a pass with two row blocks at a time; 674 us
+// with one at a time (a reduction costs more than it gains there), 672 us with three and one,
+// 650 us if the three row blocks of the fused q, k, v are split as well.
+constexpr int kEarlyRows = 2, kEarlyMinBlocks = 4;
 // A ring slot also has room for the 256 values of x that its unit multiplies (512 bytes): they are
 // requested one unit ahead, in front of the weight loads issued at the same time, and in the order
 // of the wave's loads they arrive before that unit -- no wait for x drains the ring.
@@ -68,7 +77,9 @@ struct FlowEntry {  // what the kernel needs of an entry, in LDS
 static_assert(sizeof(FlowEntry) == 64 && offsetof(FlowEntry, blob) == 16, "entry cache layout");
 struct FlowHot {  // the first 16 bytes of a FlowEntry, wave-uniform
   int k_in, x_word, nrb, x_src, x_id, m_rows;
+  int pr;  // row blocks per pass
 };
+constexpr int kEarlyBit = 0x40;  // in the m_rows byte: kEarlyRows row blocks per pass
 
 struct FlowControl {
   unsigned deposited[2];  // mailbox deposits into the set since it was last emptied
@@ -137,7 +148,8 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     c.x_src = plan->x_src[i];
     const int rb = (e.n_out + 15) >> 4;
     c.nrb = (short)(rb > b ? (rb - b + G - 1) / G : 0);
-    c.m_rows = (char)e.m_rows;
+    const bool early = plan->ex_word[i] >= 0 && c.nrb >= kEarlyMinBlocks;
+    c.m_rows = (char)(e.m_rows | (early ? kEarlyBit : 0));
     c.act = (char)e.activation;
     c.x_id = plan->x_id[i];
     c.pad[0] = c.pad[1] = 0;
@@ -197,14 +209,15 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     h.nrb = (short)(z & 0xFFFF);
     h.x_src = (short)(z >> 16);
     h.x_id = (short)(w & 0xFFFF);
-    h.m_rows = (signed char)((w >> 16) & 0xFF);
+    h.m_rows = (w >> 16) & 0x3F;
+    h.pr = ((w >> 16) & kEarlyBit) ? kEarlyRows : kFlowPR;
     return h;
   };
 
   // ---- the producer: walks this wave's units D ahead of the consumer; all of it wave-uniform
   struct Walk {
     int d, pass, hcp, j;  // entry, pass of row blocks, this wave's how-manieth 256-feature piece, row block in pass
-    int nrb, n_hc, nj, chunks;
+    int nrb, n_hc, nj, chunks, pr;
     const char *blob;
   };
   auto enter = [&](Walk &w) {  // first unit of entry w.d (n_hc == 0 or nrb == 0: none)
@@ -217,7 +230,8 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     w.chunks = k_in >> 9;
     const int pieces = k_in >> 8;
     w.n_hc = wave < pieces ? (pieces - wave + kFlowWaves - 1) / kFlowWaves : 0;
-    w.nj = min(PR, w.nrb);
+    w.pr = h.pr;
+    w.nj = min(w.pr, w.nrb);
     w.blob = uni_ptr(cache[w.d].blob);
   };
   auto next_entry = [&](Walk &w) {
@@ -232,7 +246,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     if (++w.hcp < w.n_hc) return;
     w.hcp = 0;
     ++w.pass;
-    w.nj = min(PR, w.nrb - w.pass * PR);
+    w.nj = min(w.pr, w.nrb - w.pass * w.pr);
     if (w.nj > 0) return;
     next_entry(w);
   };
@@ -255,7 +269,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         : "memory");
   };
   auto issue = [&](const Walk &w, int slot) {
-    const int64_t block = (int64_t)(b + (w.pass * PR + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
+    const int64_t block = (int64_t)(b + (w.pass * w.pr + w.j) * G) * w.chunks + (wave >> 1) + 8 * w.hcp;
     const char *src = w.blob + block * (2 * kUnitBytes) + hpar * 2048;
     const uint32_t dst = ring_rd + (uint32_t)slot * kSlot;
     asm volatile(
@@ -335,7 +349,8 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
   };
   // nothing can have arrived from everywhere before this workgroup's own share (if it has one) is stored
   auto wait_own_share = [&](int x_src) {
-    if (uni(cache[x_src].nrb) > 0)
+    // (an entry that passes its results on in parts has what this wave needs before its last part)
+    if (uni(cache[x_src].nrb) > 0 && !(uni((int)cache[x_src].m_rows) & kEarlyBit))
       while (lds_load(&ctl->stored) <= (unsigned)x_src && !lds_load(&ctl->failed)) __builtin_amdgcn_s_sleep(1);
   };
 
@@ -439,9 +454,10 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
     const int active_waves = min(kFlowWaves, pieces);
     const int x_word = hot.x_word, x_src = hot.x_src, x_id = hot.x_id;
     const char *const xrow = x_word >= 0 ? reinterpret_cast<const char *>(ex16 + x_word) : uni_ptr(cache[d].x);
-    for (int pass = 0; pass * PR < nrb; ++pass, ++q) {
+    const int pr = hot.pr;
+    for (int pass = 0; pass * pr < nrb; ++pass, ++q) {
       if (n_hc == 0) continue;
-      const int nj = min(PR, nrb - pass * PR);
+      const int nj = min(pr, nrb - pass * pr);
       float tot[PR][MC];
 #pragma unroll
       for (int j = 0; j < PR; ++j)
@@ -480,7 +496,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
           if (j + 1 < nj) {
           } else if (hcp + 1 < n_hc) {
             nx_hc = hc + kFlowWaves;
-          } else if ((pass + 1) * PR < nrb) {
+          } else if ((pass + 1) * pr < nrb) {
             if (n_hc > 1) nx_hc = wave;
           } else if (d + 1 < n_entries) {
             const FlowHot next = uniform_hot(hot_ahead);
@@ -562,7 +578,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         unsigned short *y = reinterpret_cast<unsigned short *>(const_cast<char *>(uni_ptr(cache[d].y)));
         const half_t *out_bias = reinterpret_cast<const half_t *>(uni_ptr(cache[d].out_bias));
         const int j = ((kc & 1) << 1) | (kc >> 1);
-        const int row = (b + (pass * PR + j) * G) * 16 + n;
+        const int row = (b + (pass * pr + j) * G) * 16 + n;
 #pragma unroll
         for (int e = 0; e < MC; ++e) {
           float sum = 0.f;
@@ -586,7 +602,7 @@ __device__ __forceinline__ void flow_body(const Entry *__restrict__ entries, int
         if (lane == 0) {
           __hip_atomic_store(&ctl->deposited[set], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
           __hip_atomic_store(&ctl->reduced[set], use + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          if ((pass + 1) * PR >= nrb)  // the entry's last pass in this workgroup
+          if ((pass + 1) * pr >= nrb)  // the entry's last pass in this workgroup
             // (a maximum: the wave that finishes the next entry may get here first)
             __hip_atomic_fetch_max(&ctl->stored, (unsigned)d + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
