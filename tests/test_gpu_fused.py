@@ -259,6 +259,41 @@ def test_gemv_sequence_chained_entries(hip, device, oracle, m_rows):
             x_prev = yy
 
 
+def test_gemv_sequence_results_passed_on_in_parts(hip, device, oracle):
+    """Batch 1, streaming layout, every dependency carried by data: the launch runs on the data-flow
+    kernel, where an entry that a later entry reads and that has four row blocks or more in a
+    workgroup publishes its results two row blocks at a time.  The producers here have several
+    pieces of x per wave (k_in 8192), five row blocks in every workgroup (20480 rows: passes of 2,
+    2, 1) and five in some workgroups and four in the others (16896 rows); every link of the chain
+    is checked against the oracle applied to what the device fed it."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    shapes = [(16384, 8192), (1024, 16384), (20480, 1024), (512, 20480), (4096, 512), (16896, 4096), (256, 16896)]
+    seq, refs, _ = _sequence_case(hip, device, oracle, shapes, 1, chained=True, seed=77)
+    flow, outs = GemvSequence(device), []
+    for i, (x, packed, scale, bias, y, ob) in enumerate(seq.keep):
+        y2 = torch.full_like(y, float("nan"))
+        flow.add(outs[-1] if i > 0 else x, prepack_gemv(packed, scale, bias), None, None, y2, ob, wait_previous=i > 0)
+        outs.append(y2)
+    for _ in range(3):
+        for y in outs:
+            y.fill_(float("nan"))
+        flow.run()
+        torch.cuda.synchronize()
+        assert int(flow.status.item()) == 0
+        x_prev = None
+        for i, y in enumerate(outs):
+            yy = y.cpu().numpy()
+            assert np.isfinite(yy).all(), i
+            if i == 0:
+                assert_close(yy, refs[0])
+            else:
+                e = seq.keep[i]
+                w_dec = oracle.np_decompress(e[1].cpu().numpy(), e[2].cpu().numpy(), e[3].cpu().numpy())
+                assert_close(yy, oracle.np_linear(x_prev, w_dec, None if e[5] is None else e[5].cpu().numpy()), i)
+            x_prev = yy
+
+
 @pytest.mark.parametrize("m_rows,chained", [(1, False), (2, False), (4, False), (1, True), (4, True)])
 def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
     """Weights in the streaming layout of gq_gemv_prepack_f16 give what the same sequence gives on
