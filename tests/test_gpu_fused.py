@@ -270,10 +270,12 @@ def test_gemv_sequence_results_passed_on_in_parts(hip, device, oracle):
 
     shapes = [(16384, 8192), (1024, 16384), (20480, 1024), (512, 20480), (4096, 512), (16896, 4096), (256, 16896)]
     seq, refs, _ = _sequence_case(hip, device, oracle, shapes, 1, chained=True, seed=77)
+    acts = [None, None, "gelu_tanh", None, None, "relu", None]  # (on two of the entries that publish in parts)
     flow, outs = GemvSequence(device), []
     for i, (x, packed, scale, bias, y, ob) in enumerate(seq.keep):
         y2 = torch.full_like(y, float("nan"))
-        flow.add(outs[-1] if i > 0 else x, prepack_gemv(packed, scale, bias), None, None, y2, ob, wait_previous=i > 0)
+        flow.add(outs[-1] if i > 0 else x, prepack_gemv(packed, scale, bias), None, None, y2, ob, wait_previous=i > 0,
+                 activation=acts[i])
         outs.append(y2)
     for _ in range(3):
         for y in outs:
@@ -290,7 +292,7 @@ def test_gemv_sequence_results_passed_on_in_parts(hip, device, oracle):
             else:
                 e = seq.keep[i]
                 w_dec = oracle.np_decompress(e[1].cpu().numpy(), e[2].cpu().numpy(), e[3].cpu().numpy())
-                assert_close(yy, oracle.np_linear(x_prev, w_dec, None if e[5] is None else e[5].cpu().numpy()), i)
+                assert_close(yy, oracle.np_linear(x_prev, w_dec, None if e[5] is None else e[5].cpu().numpy(), acts[i]), i)
             x_prev = yy
 
 
