@@ -31,6 +31,13 @@
 // order (0,4,1,5,2,6,3,7) in which the raw codes of a 32-bit word come out.  A wave polls exactly
 // the 256 features it multiplies, so a dependency is between 16 producing workgroups and one wave,
 // not a barrier of the device; nothing is reported, counted or flushed.
+//
+// What a dependency costs is decided by how early its data is published, not by how fast it is
+// polled: a result travels about 2 us, the waves of a workgroup finish an entry over about 4 us,
+// and a wave that finds its x missing is sent on at another time than its neighbours.  So an
+// entry that a later one reads publishes its first row blocks while its last ones still stream
+// (kEarlyRows below), and the entries of a layer are best ordered so that every reader has
+// another entry's worth of units between it and its producer.
 #include "gq_gemv_sequence.h"
 
 namespace gq {
