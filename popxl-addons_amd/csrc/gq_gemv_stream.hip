@@ -871,80 +871,137 @@ bool overlap(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes) {
 }
 
 // The plan of one launch (entries e[0..n), `first` entries of the sequence precede them and are
-// complete when the launch starts).
+// complete when the launch starts; the launch runs on `grid` workgroups).
 //
 // Entry i reads its x through the exchange when x lies inside the results of an earlier entry p of
-// the launch (the latest one that writes any of it) and waiting for the tags is all the
-// synchronisation the entry needs:
-//   * it waits for nothing past p (wait_entries <= p + 1): once every workgroup has delivered its
-//     share of p, every workgroup has also finished reading the inputs of all entries up to p (a
-//     wave works through the entries in order), which is what a declared wait protects when
-//     buffers are re-used;
+// the launch (the latest one that writes any of it) -- or, at batch 1, inside the results of several
+// earlier entries that lie end to end in memory, each the latest to write its part -- and waiting
+// for the tags is all the synchronisation the entry needs:
+//   * what it declares to wait for is covered by the arrival of x.  Once every workgroup has
+//     delivered its share of a producer q, every workgroup has also finished reading the inputs of
+//     all entries up to q (a wave works through the entries in order) -- provided every workgroup
+//     HAS a share of q, that is, q has at least one row block per workgroup.  So either the entry
+//     waits for nothing past such a producer (wait_entries <= q + 1), or none of the entries it
+//     waits for reads memory that this entry's y overwrites (then the declared wait orders nothing
+//     but the arrival of x);
 //   * out_bias is not a result of this launch, and results of the launch that y overwrites were
 //     written with the same base and shape (then the same lane of the same workgroup wrote them, in
 //     program order);
 //   * the x chunks of a wave fit its stage at once (one phase, or all phases together), x starts
-//     on a 16-byte unit of the producer's results, and the exchange has room for the producer.
+//     on a 16-byte unit of the first producer's results, and the exchange has room for the
+//     producers, end to end like their results.
 // Any other entry that reads results of this launch (x or out_bias) waits for the reported
 // completion of their producer, whatever it declares: reported completion is what makes plain
 // loads see them.
 // any_fit: the consumer has no stage that the x chunks must fit (the data-flow kernel).
-void plan_launch(const gq_gemv_desc *e, int n, int64_t first, bool any_fit, SequencePlan &plan) {
-  bool tagged[kMaxEntries];
+void plan_launch(const gq_gemv_desc *e, int n, int64_t first, bool any_fit, int grid, SequencePlan &plan) {
+  constexpr int kMaxProducers = 4;
+  struct Sources {
+    int count;
+    int16_t entry[kMaxProducers];  // in the order of their results in memory
+  };
+  static thread_local Sources sources[kMaxEntries];
   int64_t used_words = 0;
   plan.uses_exchange = 0;
   plan.exchange_values = 0;
+  auto y_bytes_of = [&](int j) { return (int64_t)e[j].m_rows * e[j].n_out * 2; };
   for (int i = 0; i < n; ++i) {
     plan.ex_word[i] = plan.x_word[i] = -1;
     plan.x_src[i] = -1;
-    tagged[i] = false;
+    Sources &from = sources[i];
+    from.count = 0;
     const gq_gemv_desc &d = e[i];
     int need = (int)(d.wait_entries > first ? d.wait_entries - first : 0);
     const int64_t x_bytes = (int64_t)d.m_rows * d.k_in * 2, y_bytes = (int64_t)d.m_rows * d.n_out * 2;
     int src = -1, bias_src = -1;
     bool same_owner = true;
     for (int j = i - 1; j >= 0; --j) {
-      const int64_t yj_bytes = (int64_t)e[j].m_rows * e[j].n_out * 2;
-      if (src < 0 && overlap(d.x, x_bytes, e[j].y, yj_bytes)) src = j;
-      if (bias_src < 0 && d.out_bias && overlap(d.out_bias, (int64_t)d.n_out * 2, e[j].y, yj_bytes)) bias_src = j;
-      if (overlap(d.y, y_bytes, e[j].y, yj_bytes) && !(e[j].y == d.y && e[j].n_out == d.n_out && e[j].m_rows == d.m_rows))
+      if (src < 0 && overlap(d.x, x_bytes, e[j].y, y_bytes_of(j))) src = j;
+      if (bias_src < 0 && d.out_bias && overlap(d.out_bias, (int64_t)d.n_out * 2, e[j].y, y_bytes_of(j))) bias_src = j;
+      if (overlap(d.y, y_bytes, e[j].y, y_bytes_of(j)) && !(e[j].y == d.y && e[j].n_out == d.n_out && e[j].m_rows == d.m_rows))
         same_owner = false;
     }
     if (src >= 0) {
-      const gq_gemv_desc &p = e[src];
-      const int64_t off = (const char *)d.x - (const char *)p.y;
+      // the producers of x, from its first byte on: each the latest entry that writes the byte
+      // where the one before ends, and nothing later writes into its part
+      const char *at = (const char *)d.x, *const end = at + x_bytes;
+      bool whole = true;
+      int latest = -1;
+      while (at < end && whole) {
+        int p = -1;
+        for (int j = i - 1; j >= 0 && p < 0; --j)
+          if ((const char *)e[j].y <= at && at < (const char *)e[j].y + y_bytes_of(j)) p = j;
+        whole = p >= 0 && from.count < kMaxProducers;
+        if (!whole) break;
+        const char *p_end = (const char *)e[p].y + y_bytes_of(p);
+        const char *part_end = p_end < end ? p_end : end;
+        for (int j = p + 1; j < i && whole; ++j) whole = !overlap(at, part_end - at, e[j].y, y_bytes_of(j));
+        // several producers: batch 1 only (rows of x would not be contiguous otherwise), each but
+        // the first read from its first result on
+        if (from.count > 0 || part_end < end) whole = whole && d.m_rows == 1 && e[p].m_rows == 1;
+        if (from.count > 0) whole = whole && at == (const char *)e[p].y;
+        from.entry[from.count++] = (int16_t)p;
+        if (p > latest) latest = p;
+        at = part_end;
+      }
+      const int64_t off = (const char *)d.x - (const char *)e[from.entry[0]].y;
       const int phases = (d.k_in + 4095) / 4096;
       const bool fits = any_fit || phases == 1 || (int64_t)phases * d.m_rows * 1024 <= kStageBytes;
-      tagged[i] = off >= 0 && off + x_bytes <= (int64_t)p.m_rows * p.n_out * 2 && off % 16 == 0 && fits && need <= src + 1 &&
-                  bias_src < 0 && same_owner;
-      if (tagged[i]) plan.x_src[i] = (int16_t)src;
-      else if (need < src + 1) need = src + 1;
+      // what the declared wait asks for beyond the arrival of x
+      bool covered = need == 0;
+      for (int s = 0; s < from.count && whole && !covered; ++s) {
+        const int q = from.entry[s];
+        covered = need <= q + 1 && (e[q].n_out + 15) / 16 >= grid;
+      }
+      if (whole && !covered && need <= latest + 1) {
+        covered = true;  // unless an entry it waits for reads what y overwrites
+        for (int j = 0; j < need && covered; ++j)
+          covered = !overlap(d.y, y_bytes, e[j].x, (int64_t)e[j].m_rows * e[j].k_in * 2) &&
+                    !(e[j].out_bias && overlap(d.y, y_bytes, e[j].out_bias, (int64_t)e[j].n_out * 2));
+      }
+      const bool tagged = whole && off % 16 == 0 && fits && covered && bias_src < 0 && same_owner;
+      if (tagged) {
+        plan.x_src[i] = (int16_t)latest;
+      } else {
+        from.count = 0;
+        if (need < src + 1) need = src + 1;
+      }
     }
     if (bias_src >= 0 && need < bias_src + 1) need = bias_src + 1;
     plan.need[i] = (int16_t)need;
   }
-  // room in the exchange, in the order the producers run
-  for (int p = 0; p < n; ++p) {
-    bool wanted = false;
-    for (int i = p + 1; i < n && !wanted; ++i) wanted = tagged[i] && plan.x_src[i] == p;
-    if (!wanted) continue;
-    const int64_t words = ((int64_t)e[p].m_rows * e[p].n_out + 63) / 64 * 64;
-    if (used_words + words > kExchangeWords) continue;
-    plan.ex_word[p] = (int32_t)used_words;
-    used_words += words;
-    plan.uses_exchange = 1;
+  // room in the exchange: the producers of one x end to end, in the order of their results
+  for (int i = 0; i < n; ++i) {
+    const Sources &from = sources[i];
+    for (int s = 0; s < from.count; ++s) {
+      const int p = from.entry[s];
+      if (plan.ex_word[p] >= 0) continue;
+      const int64_t words = ((int64_t)e[p].m_rows * e[p].n_out + 63) / 64 * 64;
+      if (used_words + words > kExchangeWords) break;
+      plan.ex_word[p] = (int32_t)used_words;
+      used_words += words;
+      plan.uses_exchange = 1;
+    }
   }
   plan.exchange_values = (int32_t)used_words;
   for (int i = 0; i < n; ++i) {
-    if (!tagged[i]) continue;
-    const int src = plan.x_src[i];
-    if (plan.ex_word[src] < 0) {  // no room: wait for the producer's reported completion instead
+    const Sources &from = sources[i];
+    if (from.count == 0) continue;
+    bool placed = true;
+    for (int s = 0; s < from.count && placed; ++s) {
+      const int p = from.entry[s];
+      placed = plan.ex_word[p] >= 0 &&
+               (s == 0 || plan.ex_word[p] == plan.ex_word[from.entry[s - 1]] + e[from.entry[s - 1]].n_out);
+    }
+    if (!placed) {  // no room, or not end to end: wait for the producers' reported completion instead
+      const int latest = plan.x_src[i];
       plan.x_src[i] = -1;
-      if (plan.need[i] < src + 1) plan.need[i] = (int16_t)(src + 1);
+      if (plan.need[i] < latest + 1) plan.need[i] = (int16_t)(latest + 1);
       continue;
     }
     plan.need[i] = 0;
-    plan.x_word[i] = plan.ex_word[src] + (int32_t)(((const char *)e[i].x - (const char *)e[src].y) / 2);
+    const int p0 = from.entry[0];
+    plan.x_word[i] = plan.ex_word[p0] + (int32_t)(((const char *)e[i].x - (const char *)e[p0].y) / 2);
   }
   for (int i = 0; i < n; ++i) {
     plan.x_id[i] = (int16_t)i;
@@ -1023,14 +1080,14 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
       const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
       SequencePlan plan;                                                                                      \
       if (kUseFlow) {                                                                                         \
-        plan_launch(host + first, n, first, true, plan);                                                      \
+        plan_launch(host + first, n, first, true, grid, plan);                                                      \
         if (flow_eligible(host + first, n, plan)) {                                                           \
           const int rc = launch_flow(host + first, device + first, n, status, words, spins, plan, grid, dev, stream); \
           if (rc != GQ_OK) return rc;                                                                         \
           continue;                                                                                           \
         }                                                                                                     \
       }                                                                                                       \
-      plan_launch(host + first, n, first, false, plan);                                                       \
+      plan_launch(host + first, n, first, false, grid, plan);                                                 \
       kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status, words, spins, plan); \
     }                                                                                                         \
   } while (0)

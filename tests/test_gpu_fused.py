@@ -296,6 +296,52 @@ def test_gemv_sequence_results_passed_on_in_parts(hip, device, oracle):
             x_prev = yy
 
 
+@pytest.mark.parametrize("streaming", [False, True])
+@pytest.mark.parametrize("hidden,ffn,inside", [(1024, 4096, 0), (1024, 4096, 1536), (4096, 16384, 0)])
+def test_gemv_sequence_x_from_several_producers(hip, device, oracle, streaming, hidden, ffn, inside):
+    """Batch 1: an entry whose x is the results of TWO earlier entries that lie end to end in memory
+    (the `up` projection's and the first third of a v|q|k projection's: the attention output and the
+    second feed-forward layer of a parallel decoder block as one product over [up | v]).  It starts
+    `inside` values into the first producer's results.  Two layers, the second reading the first's
+    output; every entry is checked against the oracle applied to what the device fed it."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    rng = np.random.default_rng(hidden + inside)
+    seq, checks = GemvSequence(device), []
+    x = to_dev(activations(1, hidden, 3), device)
+
+    def entry(x_in, n_out, y, activation=None):
+        k_in = x_in.shape[1]
+        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        dev = tuple(to_dev(a, device) for a in (packed, scale, bias))
+        if streaming:
+            seq.add(x_in, prepack_gemv(*dev), None, None, y, activation=activation)
+        else:
+            seq.add(x_in, *dev, y, activation=activation)
+        checks.append((x_in, oracle.np_decompress(packed, scale, bias), y, activation))
+
+    outs = []
+    for layer in range(2):
+        both = torch.full((1, ffn + 3 * hidden), float("nan"), dtype=torch.float16, device=device)
+        y = torch.full((1, hidden), float("nan"), dtype=torch.float16, device=device)
+        entry(x, ffn, both[:, :ffn], "gelu_tanh")
+        entry(x, 3 * hidden, both[:, ffn:])
+        entry(both[:, inside:ffn + hidden], hidden, y)
+        outs += [both, y]
+        x = y
+    for _ in range(3):
+        for t in outs:
+            t.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        for i, (x_in, w_dec, y, activation) in enumerate(checks):
+            yy = y.cpu().numpy()
+            assert np.isfinite(yy).all(), i
+            assert_close(yy, oracle.np_linear(x_in.cpu().numpy(), w_dec, None, activation), i)
+
+
 @pytest.mark.parametrize("m_rows,chained", [(1, False), (2, False), (4, False), (1, True), (4, True)])
 def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
     """Weights in the streaming layout of gq_gemv_prepack_f16 give what the same sequence gives on
