@@ -264,7 +264,8 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     return r
 
 
-FLOW_KERNEL_MODES = ("sequence_decoder_data_flow_streaming_layout", "sequence_no_waits_streaming_layout")
+FLOW_KERNEL_MODES = ("sequence_decoder_data_flow_streaming_layout", "sequence_decoder_data_flow_joint_output_streaming_layout",
+                     "sequence_no_waits_streaming_layout")
 
 
 def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, ffn=16384, modes=None):
@@ -404,18 +405,46 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             last = seq.add(v_rows(y_qkv), *w_o, y_o2[layer % 2], None, wait_for=a)
             h = y_o2[layer % 2]
 
+    # The parallel block as the model computes it: the next layer reads attention output PLUS
+    # feed-forward output, h' = W_o v + W_down up, which is ONE product [W_down | W_o] [up ; v] with
+    # the two weights side by side along their input features and x = the results of `up` and of the
+    # first third of a v|q|k projection, end to end in memory (batch 1: rows of x must be
+    # contiguous).  Three entries per layer, 84 per pass, the same weight bytes; every entry reads
+    # what earlier entries wrote, and the step to the next layer waits for all of the layer.
+    joint = None
+    if m_rows == 1 and (modes is None or "sequence_decoder_data_flow_joint_output_streaming_layout" in modes):
+        joint = {"w": [], "plain": None, "y": [torch.empty((1, hidden), dtype=torch.float16, device=device) for _ in range(2)],
+                 "both": torch.empty((1, ffn + 3 * hidden), dtype=torch.float16, device=device)}
+        for layer in range(n_layers):
+            q, k, v, o, up, down = (mats[layer * 6 + role][2:] for role in range(6))
+            vqk = tuple(torch.cat([v[part], q[part], k[part]], dim=0).contiguous() for part in range(3))
+            out = tuple(torch.cat([down[part], o[part]], dim=1).contiguous() for part in range(3))
+            joint["w"].append((prepacked[layer][2], hip.prepack_gemv(*vqk), hip.prepack_gemv(*out)))
+            if layer == n_layers - 1:
+                joint["plain"] = (up, vqk, out)
+
+    def data_flow_joint_output(seq):
+        h, last = h0, None
+        for layer in range(n_layers):
+            w_up, w_vqk, w_out = joint["w"][layer]
+            seq.add(h, w_up, None, None, joint["both"][:, :ffn], None, wait_for=last)
+            a = seq.add(h, w_vqk, None, None, joint["both"][:, ffn:], None, wait_for=last)
+            h = joint["y"][layer % 2]
+            last = seq.add(joint["both"][:, : ffn + hidden], w_out, None, None, h, None, wait_for=a)
+
     for mode, fill in (("sequence_sequential_block", sequential), ("sequence_parallel_block", parallel),
                        ("sequence_parallel_block_fused_qkv", parallel_fused_qkv),
                        ("sequence_parallel_block_fused_qkv_ffn_first", parallel_fused_qkv_ffn_first),
                        ("sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", parallel_fused_qkv_ffn_first_streaming),
                        ("sequence_decoder_data_flow", lambda seq: data_flow(seq, streaming=False)),
                        ("sequence_decoder_data_flow_streaming_layout", data_flow),
+                       ("sequence_decoder_data_flow_joint_output_streaming_layout", data_flow_joint_output),
                        ("sequence_no_waits", free), ("sequence_no_waits_streaming_layout", free_streaming)):
-        if modes is not None and mode not in modes:
+        if (modes is not None and mode not in modes) or ("joint_output" in mode and joint is None):
             continue
         seq = hip.GemvSequence(device)
         fill(seq)
-        for y in ys + [y_qkv] + y_o2:
+        for y in ys + [y_qkv] + y_o2 + ([joint["both"]] + joint["y"] if joint else []):
             y.fill_(float("nan"))
         ms = time_launches(lambda _: seq.run(), passes, warmup)
         torch.cuda.synchronize()
@@ -430,7 +459,18 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         # equals single-call GEMVs on the same weights and the inputs the device had
         worst = 0.0
         last = (n_layers - 1) * 6
-        if "data_flow" in mode:
+        if "joint_output" in mode:
+            both, h_last = joint["both"], joint["y"][(n_layers - 2) % 2]
+            singles = ((h_last, joint["plain"][0], both[:, :ffn]), (h_last, joint["plain"][1], both[:, ffn:]),
+                       (both[:, : ffn + hidden], joint["plain"][2], joint["y"][(n_layers - 1) % 2]))
+            checks = ()
+            for x_in, (p, s, b), y in singles:
+                ref = torch.empty_like(y)
+                hip.call("gq_gemv_f16", x_in.data_ptr(), 1, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
+                         y.shape[1], x_in.shape[1], GROUP, stream_handle())
+                torch.cuda.synchronize()
+                worst = max(worst, ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item())
+        elif "data_flow" in mode:
             h_last = y_o2[(n_layers - 2) % 2]
             checks = ((3, v_rows(y_qkv), y_o2[(n_layers - 1) % 2]), (4, h_last, ys[4]), (5, ys[4], ys[5]))
         else:

@@ -189,6 +189,40 @@ class LinearGQ:
             fused.variables.insert("bias", Variable("bias", torch.cat([l.variables.bias.data for l in layers]).contiguous()))
         return fused
 
+    @classmethod
+    def fuse_inputs(cls, layers):
+        """One layer computing the SUM of `layers`, each applied to its own slice of the input
+        features: y = sum(l_i(x_i)) for x = cat([x_i], -1) (e.g. the attention output projection and
+        the second feed-forward layer of a parallel decoder block, whose results are added: one
+        product over [attention values ; feed-forward activations]).  The weights lie side by side
+        along their input features: the variables stack along the group axis for dim=0 and along
+        their first axis for dim=-1 / 1; the additive biases are summed in float32.  All layers
+        must agree in dim, group_size, bias and output width.  The new layer owns its variables.
+        """
+        import torch
+
+        layers = list(layers)
+        if not layers:
+            raise ValueError("LinearGQ.fuse_inputs: no layers")
+        first = layers[0]
+        for layer in layers:
+            if layer.variables is None:
+                raise ValueError("LinearGQ.fuse_inputs: every layer needs its variables (build it or call init_variables)")
+            if (layer.dim == 0) != (first.dim == 0):
+                raise NotImplementedError("LinearGQ.fuse_inputs: layers grouped along different axes do not stack")
+            if layer.group_size != first.group_size or layer.bias != first.bias or layer.out_features != first.out_features:
+                raise ValueError("LinearGQ.fuse_inputs: layers differ in group_size, bias or output features")
+        fused = cls(first.out_features, bias=first.bias, group_size=first.group_size, dim=first.dim)
+        axis = 1 if first.dim == 0 else 0
+        names = ["weight_compressed", "weight_decompression_scale", "weight_decompression_bias"]
+        fused.variables = NamedTensors(
+            **{n: Variable(n, torch.cat([l.variables[n].data for l in layers], dim=axis).contiguous()) for n in names}
+        )
+        if first.bias:
+            total = sum(l.variables.bias.data.float() for l in layers).to(first.variables.bias.data.dtype)
+            fused.variables.insert("bias", Variable("bias", total.contiguous()))
+        return fused
+
     def prepacked(self):
         """The weight in the streaming layout that `_gq_hip.GemvSequence.add` accepts in place of the
         three variables (a device copy made by gq_gemv_prepack_f16; dim=0, group_size 64 and input

@@ -207,6 +207,33 @@ def test_fused_qkv_equals_separate_projections(hip, device, batch):
     assert_bits_equal(fused(x).cpu().numpy(), want.cpu().numpy())
 
 
+@pytest.mark.parametrize("dim", [0, -1])
+@pytest.mark.parametrize("batch", [1, 40])
+def test_fused_inputs_equal_the_sum_of_the_layers(hip, device, dim, batch):
+    """Two layers whose results are added (each reading its own input): their weights side by side
+    along the input features give one layer on the concatenated inputs.  The sum is then taken in
+    float32 inside the kernel instead of on two float16 results."""
+    out_features, group_size = 384, 64
+    torch.manual_seed(4)
+    layers, xs = [], []
+    for in_features in (512, 1024):
+        nn_layer = torch.nn.Linear(in_features, out_features)
+        layer = LinearGQ(out_features, bias=True, group_size=group_size, dim=dim)
+        variables = layer.init_variables(in_features, torch.float16, device)
+        layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=dim))
+        layers.append(layer)
+        xs.append(torch.randn((batch, in_features), device=device, dtype=torch.float16))
+    fused = LinearGQ.fuse_inputs(layers)
+    assert fused.out_features == out_features
+    got = fused(torch.cat(xs, dim=-1)).float()
+    want = sum(layer(x).float() for layer, x in zip(layers, xs))
+    assert ((got - want).abs().max() / want.abs().max()).item() <= 2e-3
+    other = LinearGQ(out_features + 64, bias=True, group_size=group_size, dim=dim)
+    other.init_variables(512, torch.float16, device)
+    with pytest.raises(ValueError):
+        LinearGQ.fuse_inputs([layers[0], other])
+
+
 def test_prepacked_layer_in_a_sequence(hip, device):
     """LinearGQ.prepacked(): the layer's weight in the streaming layout, run as entries of a GEMV
     sequence (up-projection with GELU, then the down-projection that waits for it), gives what the

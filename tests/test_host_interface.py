@@ -196,6 +196,41 @@ def test_linear_gq_variables_and_mapping():
     assert "bias" not in LinearGQ(8, bias=False, group_size=4).init_variables(8, torch.float16, "cpu")
 
 
+@pytest.mark.parametrize("dim", [0, -1])
+def test_linear_gq_fused_variables(oracle, dim):
+    """LinearGQ.fuse (outputs side by side) and LinearGQ.fuse_inputs (inputs side by side, results
+    added): the stacked variables decompress to the layers' [in, out] weights laid side by side."""
+    torch.manual_seed(1)
+
+    def layer_of(n_in, n_out):
+        nn_layer = torch.nn.Linear(n_in, n_out, bias=True)
+        layer = LinearGQ(n_out, bias=True, group_size=16, dim=dim)
+        v = layer.init_variables(n_in, torch.float16, "cpu")
+        layer.load_weights(LinearGQ.torch_mapping(v, nn_layer, dtype=torch.float16, group_size=16, dim=dim))
+        return layer
+
+    def weight_in_out(layer):
+        v = layer.variables
+        w = oracle.np_decompress(*(v[n].data.numpy() for n in ("weight_compressed", "weight_decompression_scale", "weight_decompression_bias")))
+        return w.T if dim == 0 else w  # dim=0 keeps [out, in]
+
+    a, b = layer_of(64, 48), layer_of(64, 80)
+    wide = LinearGQ.fuse([a, b])
+    assert wide.out_features == 128
+    assert np.array_equal(weight_in_out(wide), np.concatenate([weight_in_out(a), weight_in_out(b)], axis=1))
+    assert np.array_equal(wide.variables.bias.data.numpy(), np.concatenate([a.variables.bias.data.numpy(), b.variables.bias.data.numpy()]))
+    c, d = layer_of(64, 48), layer_of(96, 48)
+    deep = LinearGQ.fuse_inputs([c, d])
+    assert deep.out_features == 48
+    assert np.array_equal(weight_in_out(deep), np.concatenate([weight_in_out(c), weight_in_out(d)], axis=0))
+    total = (c.variables.bias.data.float() + d.variables.bias.data.float()).to(torch.float16)
+    assert np.array_equal(deep.variables.bias.data.numpy(), total.numpy())
+    with pytest.raises(ValueError):
+        LinearGQ.fuse_inputs([a, b])  # other output widths
+    with pytest.raises(ValueError):
+        LinearGQ.fuse_inputs([])
+
+
 def test_linear_gq_misuse():
     with pytest.raises(ZeroDivisionError):  # group_size left at its default 0 (linear_gq.py:25,73)
         LinearGQ(8).init_variables(8, torch.float16, "cpu")
