@@ -151,9 +151,16 @@ __device__ __forceinline__ void compress_item(const uint4_t (&q)[V], int64_t ite
   }
   // (Collecting the statistics of four groups in one lane for 8-byte stores was measured: the
   // shuffles cost what the wider stores save.)
-  if (live && (item & (LANES - 1)) == 0) {
-    scale[item / LANES] = sc;
-    bias[item / LANES] = lo;
+  if (LANES == 1) {
+    if (live) {
+      scale[item] = sc;
+      bias[item] = lo;
+    }
+  } else if (live && (item & (LANES - 1)) < 2) {
+    // the first lane of a group stores its scale, the second its bias: one store instruction for
+    // both arrays (0.15 us of 31 against one lane storing both)
+    half_t *const dst = (item & 1) ? bias : scale;
+    dst[item / LANES] = (item & 1) ? lo : sc;
   }
 }
 
