@@ -30,12 +30,23 @@ namespace {
 // GS    64 or 128: scale/bias of a chunk are fetched as one 16/8-byte load per row and the lane's
 //       value is picked with a byte permute; 0: any power-of-two group >= 32, 2-byte loads.
 // FULL  k_in is a multiple of 512 (no slot predication).
-template <int NWAVES, int R, int GS, bool FULL>
+// XM    0: the lanes of batch row m fetch that row's x themselves, 16 bytes at a time (sixteen load
+//       instructions per chunk with 4 m_rows lanes active).  > 0 (m_rows <= XM, FULL): a chunk of a
+//       batch row is 1 KiB, fetched by ONE instruction of the whole wave and handed to the row's four
+//       lanes through LDS.  Measured on 4096 x 4096: the x loads of XM = 0 cost 0.8 us of 5.9 at one
+//       batch row and 1.9 us of 7.1 at eight.
+constexpr int gemv_region_bytes(int r, int xm) { return (xm > r ? xm : r) * 1024; }
+
+template <int NWAVES, int R, int GS, bool FULL, int XM>
 __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
     int gs_shift, int act) {
-  __shared__ float4_t partial[NWAVES][R][64];
+  static_assert(XM == 0 || FULL, "staged x needs whole chunks");
+  // per wave: the x chunk of up to XM batch rows while the wave walks K, its partial sums at the end
+  constexpr int kRegion = gemv_region_bytes(R, XM);
+  extern __shared__ __attribute__((aligned(16))) char region_base[];
+  char(*const region)[kRegion] = reinterpret_cast<char(*)[kRegion]>(region_base);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kc = lane >> 4;
   const int n_slots = k_in >> 7;
@@ -60,7 +71,19 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < R; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+  // staged x: 16-byte piece p of batch row m lies at piece p ^ m of the row's KiB, so that the sixteen
+  // rows read by lanes of one slice fall on different banks
+  char *const stage = region[wave];
+  const int x_row = has_x ? r : 0;  // (columns past the batch are never stored: they may hold any row)
   for (int c = wave; c < n_chunks; c += NWAVES) {
+    uint4_t xq[XM > 0 ? XM : 1];
+    if constexpr (XM > 0) {
+#pragma unroll
+      for (int m = 0; m < XM; ++m) {
+        xq[m] = uint4_t{0u, 0u, 0u, 0u};
+        if (m < m_rows) xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + c * 512 + lane * 8);
+      }
+    }
     uint4_t wq[R][4];
     uint32_t s2[R][4], b2[R][4];  // (scale, scale) and (bias, bias) as packed fp16 pairs
     // ---- issue every load of the chunk
@@ -113,7 +136,16 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         uint4_t q = {0u, 0u, 0u, 0u};
-        if (has_x && (FULL || slot < n_slots)) q = *reinterpret_cast<const uint4_t *>(xrow + slot * 128 + s * 8);
+        if constexpr (XM > 0) {
+          if (j == 0 && s == 0) {
+#pragma unroll
+            for (int m = 0; m < XM; ++m)
+              if (m < m_rows) *reinterpret_cast<uint4_t *>(stage + m * 1024 + ((lane ^ m) & 63) * 16) = xq[m];
+          }
+          q = *reinterpret_cast<const uint4_t *>(stage + x_row * 1024 + ((j * 16 + kc * 4 + s) ^ x_row) * 16);
+        } else {
+          if (has_x && (FULL || slot < n_slots)) q = *reinterpret_cast<const uint4_t *>(xrow + slot * 128 + s * 8);
+        }
         xp[j][s] = permute_x(q);
       }
     }
@@ -129,14 +161,14 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
         }
   }
 #pragma unroll
-  for (int i = 0; i < R; ++i) partial[wave][i][lane] = acc[i];
+  for (int i = 0; i < R; ++i) *reinterpret_cast<float4_t *>(region[wave] + (i * 64 + lane) * 16) = acc[i];
   __syncthreads();
   // lane holds D[n = 4 * kc + e][m = r] of row block i
   for (int t = threadIdx.x; t < R * 64; t += NWAVES * 64) {
     const int i = t >> 6, l = t & 63;
-    float4_t sum = partial[0][i][l];
+    float4_t sum = *reinterpret_cast<const float4_t *>(region[0] + (i * 64 + l) * 16);
 #pragma unroll
-    for (int w = 1; w < NWAVES; ++w) sum += partial[w][i][l];
+    for (int w = 1; w < NWAVES; ++w) sum += *reinterpret_cast<const float4_t *>(region[w] + (i * 64 + l) * 16);
     const int m = l & 15;
     if (m < m_rows) {
       const int n0 = ((int)blockIdx.x * R + i) * 16 + 4 * (l >> 4);
@@ -207,11 +239,12 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream) {
-  // Large weights at small batches go through the persistent kernel as a sequence of one: its
-  // pipelined rings beat the one-shot kernel below once the weight is tens of megabytes (measured:
-  // 16384x4096 at one row 14.5 -> 11.7 us). With 3 or 4 rows that holds only for the wide outputs
-  // (4096x16384: 17.2 us one-shot, 18.0 us streamed).
-  const bool large = n_out * k_in >= ((int64_t)24 << 20) && (m_rows <= 2 || n_out >= 8192);
+  // Large weights with rows of up to 4096 features go through the persistent kernel at small
+  // batches, as a sequence of one: its pipelined rings beat the one-shot kernel below there
+  // (measured: 16384x4096 at one row 12.6 -> 11.5 us, 32768x4096 22.3 -> 18.1 us; with 3 or 4 rows
+  // only for the wide outputs).  With longer rows a wave of the one-shot kernel has several chunks
+  // to overlap and wins (4096x16384 at one row: 12.0 against 14.5 us; 8192x8192: 13.3 against 14.1).
+  const bool large = n_out * k_in >= ((int64_t)24 << 20) && k_in < 8192 && (m_rows <= 2 || n_out >= 8192);
   if (large && m_rows <= 4) {
     const int rc =
         launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
@@ -238,24 +271,46 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),                    \
       reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act
-#define GQ_GEMV_LAUNCH(NW, R, GS, FULL) \
-  gemv_mfma_kernel<NW, R, GS, FULL><<<dim3(blocks), dim3(NW * 64), 0, stream>>>(GQ_GEMV_ARGS)
-#define GQ_GEMV_BY_R(NW, GS, FULL)                      \
-  do {                                                  \
-    if (r == 4) GQ_GEMV_LAUNCH(NW, 4, GS, FULL);        \
-    else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL);   \
-    else GQ_GEMV_LAUNCH(NW, 1, GS, FULL);               \
+#define GQ_GEMV_LAUNCH(NW, R, GS, FULL, XM)                                                              \
+  do {                                                                                                    \
+    constexpr int lds_bytes = NW * gemv_region_bytes(R, XM);                                              \
+    static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                \
+    if (lds_bytes > 64 * 1024) { /* beyond the default limit of a launch */                               \
+      constexpr int kMaxDevices = 64;                                                                     \
+      static bool configured[kMaxDevices] = {false};                                                      \
+      int dev = 0;                                                                                        \
+      if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return GQ_ERR_NO_DEVICE;     \
+      if (!configured[dev]) {                                                                             \
+        const hipError_t e = hipFuncSetAttribute(                                                         \
+            reinterpret_cast<const void *>(gemv_mfma_kernel<NW, R, GS, FULL, XM>),                        \
+            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                                       \
+        if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));        \
+        configured[dev] = true;                                                                           \
+      }                                                                                                   \
+    }                                                                                                     \
+    gemv_mfma_kernel<NW, R, GS, FULL, XM><<<dim3(blocks), dim3(NW * 64), lds_bytes, stream>>>(GQ_GEMV_ARGS); \
   } while (0)
-    if (gs_mode == 64) {
-      if (r == 1 && k_in >= 8192) GQ_GEMV_LAUNCH(16, 1, 64, true);
-      else GQ_GEMV_BY_R(8, 64, true);
-    } else if (gs_mode == 128) {
-      GQ_GEMV_BY_R(8, 128, true);
-    } else if (full) {
-      GQ_GEMV_BY_R(8, 0, true);
-    } else {
-      GQ_GEMV_BY_R(8, 0, false);
-    }
+#define GQ_GEMV_BY_R(NW, GS, FULL, XM)                      \
+  do {                                                      \
+    if (r == 4) GQ_GEMV_LAUNCH(NW, 4, GS, FULL, XM);        \
+    else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL, XM);   \
+    else GQ_GEMV_LAUNCH(NW, 1, GS, FULL, XM);               \
+  } while (0)
+    // whole chunks: x through LDS, one load instruction per batch row and chunk (the rows of x are
+    // 16-byte aligned then), on eight waves whatever the length of the rows (measured on 4096 x 16384:
+    // 16 waves are no faster with x staged; without, eight rows took 20.1 us against 14.7 us)
+#define GQ_GEMV_BY_M(GS)                                    \
+  do {                                                      \
+    if (m_rows == 1) GQ_GEMV_BY_R(8, GS, true, 1);          \
+    else if (m_rows <= 4) GQ_GEMV_BY_R(8, GS, true, 4);     \
+    else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, true, 8);     \
+    else GQ_GEMV_BY_R(8, GS, true, 16);                     \
+  } while (0)
+    if (gs_mode == 64) GQ_GEMV_BY_M(64);
+    else if (gs_mode == 128) GQ_GEMV_BY_M(128);
+    else if (full) GQ_GEMV_BY_M(0);
+    else GQ_GEMV_BY_R(8, 0, false, 0);
+#undef GQ_GEMV_BY_M
 #undef GQ_GEMV_BY_R
 #undef GQ_GEMV_LAUNCH
 #undef GQ_GEMV_ARGS

@@ -74,6 +74,21 @@ def test_gemv_benchmark_shapes(hip, device, oracle, n_out, k_in, m_rows):
         (8, 96, 8, 2),  # generic: k_in % 128 != 0
         (5, 12, 12, 16),  # generic: group 12
         (64, 8192, 256, 7),
+        # group 64, k_in % 512 == 0: x goes through LDS (1, 4, 8 or 16 rows), with 1, 2 or 4 row blocks per wave
+        (40, 512, 64, 1),
+        (8200, 1024, 64, 1),
+        (8200, 512, 64, 7),
+        (8200, 1536, 64, 13),
+        (16400, 512, 64, 3),
+        (16400, 1024, 64, 8),
+        (16400, 512, 64, 16),
+        (100, 8192, 64, 2),  # several chunks per wave
+        (100, 8192, 64, 11),
+        # the same with groups of 128 (8-byte scale / bias loads) and of 32 and 256 (2-byte loads)
+        (48, 1024, 128, 5),
+        (8200, 512, 128, 2),
+        (33, 512, 32, 9),
+        (16400, 1024, 256, 1),
     ],
 )
 def test_gemv_edge_shapes(hip, device, oracle, n_out, k_in, gs, m_rows):
