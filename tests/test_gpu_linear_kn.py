@@ -84,6 +84,12 @@ def test_prefill_shapes(hip, device, oracle, m_rows):
         (40, 8, 8, 16),  # generic: n_out < 32
         (50, 128, 64, 40),  # prefill, k_in % 64 != 0: generic
         (5000, 32, 32, 1),  # many K slabs for one strip
+        # groups of 64 and whole strips of 256 outputs, every batch size class, ragged K slabs
+        (7, 256, 64, 1),
+        (1001, 512, 64, 2),
+        (333, 768, 64, 4),
+        (2050, 256, 64, 7),
+        (515, 1280, 64, 13),
     ],
 )
 def test_edge_shapes(hip, device, oracle, k_in, n_out, gs, m_rows):
