@@ -96,7 +96,9 @@ int gq_decompress_f16_transposed(const uint16_t *packed, const uint16_t *scale, 
  *
  * gq_gemv_f16  decode-sized batches, 1 <= m_rows <= 16.
  * gq_gemm_f16  prefill-sized batches (any m_rows >= 1; built for m_rows >= 16).
- * gq_linear_f16 picks between them by m_rows; it is what the LinearGQ wrapper calls.
+ * gq_linear_f16 picks between them by m_rows (and, for 17 to 128 rows on large weights, runs
+ *              several GEMV launches of 16 rows each where those are faster than the GEMM's
+ *              mostly empty tiles); it is what the LinearGQ wrapper calls.
  *
  * Requirements: group_size % 4 == 0, k_in % group_size == 0.  Fast kernels need a power-of-two
  * group_size >= 32, k_in % 128 == 0 (GEMV) or % 64 == 0 (GEMM) and 16-byte aligned x / packed;

@@ -135,6 +135,10 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
   if (m_rows <= 16)
     return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
                            (hipStream_t)stream);
+  int passes_rc = GQ_OK;
+  if (gq::launch_gemv_passes(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
+                             (hipStream_t)stream, &passes_rc))
+    return passes_rc;
   return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
                          (hipStream_t)stream);
 }

@@ -40,6 +40,12 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream);
+// Batches of 17 to 128 rows as passes of the GEMV kernel over 16 rows each, where that is expected
+// to beat the GEMM kernel (whose 128 x 64 tiles are mostly empty there); false: not such a case,
+// nothing launched.
+bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                        const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                        int64_t group_size, int act, hipStream_t stream, int *rc);
 int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                              const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                              int64_t k_in, int64_t group_size, int act, hipStream_t stream);

@@ -163,6 +163,19 @@ def test_gemm_edge_shapes(hip, device, oracle, n_out, k_in, gs, m_rows):
             assert_close(y, y_ref, (entry, with_bias))
 
 
+@pytest.mark.parametrize("n_out,k_in,m_rows", [(4096, 4096, 17), (4096, 4096, 40), (4096, 4096, 64), (4096, 4096, 96),
+                                               (4096, 16384, 90), (16384, 4096, 32), (16384, 4096, 48), (4104, 4096, 33)])
+def test_linear_mid_batches(hip, device, oracle, n_out, k_in, m_rows):
+    """gq_linear_f16 between the GEMV's 16 rows and full GEMM tiles: on large weights it runs passes of
+    the GEMV kernel over 16 rows each where those are expected to beat the mostly empty GEMM tiles
+    (some of these cases), the GEMM kernel otherwise; either way the result is that of gq_gemm_f16."""
+    x, packed, scale, bias, ob, y_ref = _case(oracle, n_out, k_in, 64, m_rows, 17, True)
+    y = _call(hip, "gq_linear_f16", x, packed, scale, bias, ob, n_out, k_in, 64, device)
+    assert_close(y, y_ref, (n_out, k_in, m_rows))
+    y_gemm = _call(hip, "gq_gemm_f16", x, packed, scale, bias, ob, n_out, k_in, 64, device)
+    assert normalised_error(y, y_gemm.astype(np.float32)) <= REGRESSION_TOL
+
+
 @pytest.mark.parametrize("m_rows", [33, 70, 100, 260, 300, 1030])
 def test_gemm_every_kernel_shape(hip, device, oracle, m_rows):
     """Each tile shape of the pipelined kernel, reached by the batch size (256 x 256 from 1024 rows,
