@@ -579,8 +579,25 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
   if ((k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    if (m_rows >= 1024) return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
-    if (m_rows >= 256) return GQ_PIPE2(1, 4, 8, 1, 3, 1);   // 256 x 128, 4 waves of 256 x 32
+    // Three tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
+    // launch is as slow as its busiest compute unit: expected time = tiles per compute unit (256 of
+    // them; a last, partly filled round runs faster: fewer workgroups share memory and clocks) x
+    // time per tile, from measured times per 1024 input features with every compute unit busy:
+    //   128 x 64   8 us   (16384 x 4096 at 128 rows: 34.5 us)
+    //   256 x 128  22 us  (16384 x 4096 at 512 rows: 87 us; 16 us with an eighth of the compute units busy)
+    //   256 x 256  34 us  (two per compute unit at a time; 16384 x 4096 at 2048 rows: 271 us, at 1024 rows 140 us)
+    // Fixed thresholds on the batch alone (256 x 128 from 256 rows, 256 x 256 from 1024) left weights
+    // with 4096 outputs on 16 to 64 workgroups: 4096 x 4096 at 512 rows took 75.6 us, now 36 us.  With each
+    // shape forced in turn, this choice was the fastest or within 2 % of it for five weight shapes
+    // (16384 x 4096, 4096 x 16384, 4096 x 4096, 12288 x 4096, 8192 x 8192) at nine batches from 128 to 4096.
+    auto expected = [&](int tile_m, int tile_n, double us_per_1024) {
+      const int64_t tiles = ((m_rows + tile_m - 1) / tile_m) * ((n_out + tile_n - 1) / tile_n);
+      const int64_t full = tiles / 256, rest = tiles % 256;
+      return ((double)full + (rest ? 0.7 + 0.3 * (double)rest / 256.0 : 0.0)) * us_per_1024 * (double)k_in / 1024.0;
+    };
+    const double t_small = expected(128, 64, 8.0), t_mid = expected(256, 128, 22.0), t_large = expected(256, 256, 34.0);
+    if (t_large <= t_mid && t_large <= t_small) return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
+    if (t_mid <= t_small) return GQ_PIPE2(1, 4, 8, 1, 3, 1);                        // 256 x 128, 4 waves of 256 x 32
     // 128 x 64 (a workgroup on every compute unit at n_out = 16384), 4 waves of 64 x 32; two such
     // groups of waves split K when the K tiles divide between them (and the scale / bias dwords)
     if (k_in % 256 == 0) return GQ_PIPE2(2, 2, 2, 1, 3, 1, 2);

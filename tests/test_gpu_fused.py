@@ -176,12 +176,21 @@ def test_linear_mid_batches(hip, device, oracle, n_out, k_in, m_rows):
     assert normalised_error(y, y_gemm.astype(np.float32)) <= REGRESSION_TOL
 
 
+@pytest.mark.parametrize("n_out,k_in,m_rows", [(4104, 384, 1030), (4104, 384, 2060), (4104, 512, 300), (8200, 256, 777)])
+def test_gemm_large_tiles_on_ragged_problems(hip, device, oracle, n_out, k_in, m_rows):
+    """The tile shape is chosen by expected time (tiles per compute unit x time per tile): these ragged
+    problems are large enough for the 256 x 128 tiles (1030 rows), the 256 x 256 tiles (2060 and 777
+    rows) and 128 x 64 tiles with K split between two groups of waves (300 rows)."""
+    x, packed, scale, bias, ob, y_ref = _case(oracle, n_out, k_in, 64, m_rows, 47, True)
+    y = _call(hip, "gq_gemm_f16", x, packed, scale, bias, ob, n_out, k_in, 64, device)
+    assert_close(y, y_ref, (n_out, k_in, m_rows))
+
+
 @pytest.mark.parametrize("m_rows", [33, 70, 100, 260, 300, 1030])
 def test_gemm_every_kernel_shape(hip, device, oracle, m_rows):
-    """Each tile shape of the pipelined kernel, reached by the batch size (256 x 256 from 1024 rows,
-    256 x 128 from 256, 128 x 64 below, with K split between two groups of waves where k_in is a
-    multiple of 256), the LDS-staged tile kernel (odd number of groups per row, or scale / bias that
-    are only 2-byte aligned) and the generic kernel (group 16), on ragged problems."""
+    """Small ragged problems on the pipelined kernel's 128 x 64 tiles (with K split between two groups
+    of waves where k_in is a multiple of 256), the LDS-staged tile kernel (odd number of groups per
+    row, or scale / bias that are only 2-byte aligned) and the generic kernel (group 16)."""
     for n_out, k_in, gs in ((300, 1024, 64), (130, 448, 32), (96, 192, 64), (200, 768, 128), (72, 320, 64), (40, 96, 16)):
         x, packed, scale, bias, ob, y_ref = _case(oracle, n_out, k_in, gs, m_rows, 41, True)
         y = _call(hip, "gq_gemm_f16", x, packed, scale, bias, ob, n_out, k_in, gs, device)
