@@ -222,6 +222,21 @@ def test_linearity_at_full_size(hip, device):
         assert err <= TOL, (entry, err)
 
 
+_FULL_SIZE_WEIGHTS = {}
+
+
+def _full_size_weight(oracle, n_out, k_in, seed):
+    """(packed, scale, bias, decompressed) of a seeded N(0, 1 / k_in) weight -- a scale that keeps a
+    chain of layers at unit magnitude; made once per session (a full-size weight takes seconds to draw,
+    compress and decompress on the host, and several tests and their cases use the same ones)."""
+    key = (n_out, k_in, seed)
+    if key not in _FULL_SIZE_WEIGHTS:
+        w = np.random.default_rng(seed).normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        _FULL_SIZE_WEIGHTS[key] = (packed, scale, bias, oracle.np_decompress(packed, scale, bias))
+    return _FULL_SIZE_WEIGHTS[key]
+
+
 def _sequence_case(hip, device, oracle, shapes, m_rows, chained, seed=50):
     """Entries of the given (n_out, k_in) shapes; `chained`: entry i reads entry i-1's output."""
     from popxl_addons._gq_hip import GemvSequence
@@ -232,11 +247,8 @@ def _sequence_case(hip, device, oracle, shapes, m_rows, chained, seed=50):
     x_host = activations(m_rows, shapes[0][1], seed)
     x_dev = to_dev(x_host, device)
     for i, (n_out, k_in) in enumerate(shapes):
-        # a weight scale that keeps a chain of layers at unit magnitude
-        w = (rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in))).astype(np.float16)
-        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        packed, scale, bias, w_dec = _full_size_weight(oracle, n_out, k_in, 1000 * seed + i)
         ob = rng.normal(0, 0.1, (n_out,)).astype(np.float16) if i % 2 else None
-        w_dec = oracle.np_decompress(packed, scale, bias)
         if chained and i > 0:
             assert k_in == shapes[i - 1][0]
             x_host = refs[-1].astype(np.float16)  # what the device chain holds up to fp16 rounding
@@ -343,20 +355,18 @@ def test_gemv_sequence_x_from_several_producers(hip, device, oracle, streaming, 
     output; every entry is checked against the oracle applied to what the device fed it."""
     from popxl_addons._gq_hip import GemvSequence, prepack_gemv
 
-    rng = np.random.default_rng(hidden + inside)
     seq, checks = GemvSequence(device), []
     x = to_dev(activations(1, hidden, 3), device)
 
     def entry(x_in, n_out, y, activation=None):
         k_in = x_in.shape[1]
-        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
-        packed, scale, bias = group_quantize_compress_numpy(w, 64)
+        packed, scale, bias, w_dec = _full_size_weight(oracle, n_out, k_in, 7000 + 10 * (hidden + inside) + len(checks))
         dev = tuple(to_dev(a, device) for a in (packed, scale, bias))
         if streaming:
             seq.add(x_in, prepack_gemv(*dev), None, None, y, activation=activation)
         else:
             seq.add(x_in, *dev, y, activation=activation)
-        checks.append((x_in, oracle.np_decompress(packed, scale, bias), y, activation))
+        checks.append((x_in, w_dec, y, activation))
 
     outs = []
     for layer in range(2):
@@ -750,12 +760,10 @@ def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows
     from popxl_addons._gq_hip import GemvSequence, prepack_gemv
 
     hidden, ffn, n_layers = 4096, 16384, 3
-    rng = np.random.default_rng(500 + m_rows)
 
-    def weight(n_out, k_in):
-        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
-        packed, scale, bias = group_quantize_compress_numpy(w, 64)
-        return oracle.np_decompress(packed, scale, bias), prepack_gemv(*(to_dev(a, device) for a in (packed, scale, bias)))
+    def weight(n_out, k_in, seed):
+        packed, scale, bias, w_dec = _full_size_weight(oracle, n_out, k_in, seed)  # (the same for every case of this test)
+        return w_dec, prepack_gemv(*(to_dev(a, device) for a in (packed, scale, bias)))
 
     def out(n):
         return torch.full((m_rows, n), float("nan"), dtype=torch.float16, device=device)
@@ -763,8 +771,9 @@ def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows
     def v_rows(y_qkv):  # m_rows x 4096 contiguous values out of qkv's output, starting at its column 8192
         return y_qkv.view(-1)[2 * hidden : 2 * hidden + m_rows * hidden].view(m_rows, hidden)
 
-    weights = [{name: weight(*shape) for name, shape in (("up", (ffn, hidden)), ("qkv", (3 * hidden, hidden)),
-                                                           ("down", (hidden, ffn)), ("o", (hidden, hidden)))} for _ in range(n_layers)]
+    weights = [{name: weight(*shape, 500 + 10 * layer + i)
+                for i, (name, shape) in enumerate((("up", (ffn, hidden)), ("qkv", (3 * hidden, hidden)),
+                                                   ("down", (hidden, ffn)), ("o", (hidden, hidden))))} for layer in range(n_layers)]
     h0 = to_dev(activations(m_rows, hidden, 9), device)
 
     def build(shared_buffers):
