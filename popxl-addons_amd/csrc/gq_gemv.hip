@@ -239,12 +239,13 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream) {
-  // Large weights with rows of up to 4096 features go through the persistent kernel at small
-  // batches, as a sequence of one: its pipelined rings beat the one-shot kernel below there
-  // (measured: 16384x4096 at one row 12.6 -> 11.5 us, 32768x4096 22.3 -> 18.1 us; with 3 or 4 rows
-  // only for the wide outputs).  With longer rows a wave of the one-shot kernel has several chunks
-  // to overlap and wins (4096x16384 at one row: 12.0 against 14.5 us; 8192x8192: 13.3 against 14.1).
-  const bool large = n_out * k_in >= ((int64_t)24 << 20) && k_in < 8192 && (m_rows <= 2 || n_out >= 8192);
+  // Weights of 72 Mi elements or more with rows shorter than 8192 features go through the persistent
+  // kernel at batches up to 4, as a sequence of one: its pipelined rings beat the one-shot kernel below
+  // there (measured at one row: 20480x4096 15.1 -> 13.2 us, 24576x4096 19.7 -> 14.6 us, 32768x4096
+  // 22.6 -> 17.9 us; 16384x4096 is a tie at one row, 11.6 us, and the one-shot kernel wins at four rows,
+  // 11.6 against 12.9 us).  With longer rows a wave of the one-shot kernel has several chunks to
+  // overlap and wins (4096x16384 at one row: 12.0 against 14.5 us; 8192x8192: 13.3 against 14.1).
+  const bool large = n_out * k_in >= ((int64_t)72 << 20) && k_in < 8192;
   if (large && m_rows <= 4) {
     const int rc =
         launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
@@ -259,7 +260,19 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     const bool full = k_in % 512 == 0;
     // rows per wave: reuse the permuted x fragments as often as the row count allows while still
     // filling 256 compute units
-    const int r = row_blocks >= 1024 ? 4 : (row_blocks >= 512 ? 2 : 1);
+    // Row blocks per wave (1, 2 or 4; they re-use the x fragments): the choice that moves the fewest
+    // bytes per busy compute unit -- the weights once, x once per workgroup (out of L2: counted half),
+    // divided by the share of the compute units' turns that the workgroups fill (192 workgroups
+    // leave a quarter of the 256 compute units idle).  Measured on 12288 x 4096 at one row: 9.7 us with
+    // one row block per wave (768 workgroups), 12.5 us with two (384), 11.2 us with four (192).
+    int r = 1;
+    double best = 0;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+      const int64_t wgs = (row_blocks + cand - 1) / cand;
+      const double fill = (double)wgs / (double)((wgs + 255) / 256 * 256);
+      const double bytes = (double)n_out * k_in * 0.5625 + 0.5 * (double)wgs * m_rows * k_in * 2.0;
+      if (best == 0 || bytes / fill < best) best = bytes / fill, r = cand;
+    }
     // the GS == 64 / 128 instantiations fetch a chunk's scales and biases as one 16 / 8-byte load per
     // row: that needs the arrays aligned accordingly; otherwise the 2-byte loads of GS == 0 serve
     const uintptr_t sb_align = (uintptr_t)scale | (uintptr_t)bias;

@@ -42,20 +42,27 @@ def _call(hip, entry, x, packed, scale, bias, out_bias, n_out, k_in, gs, device)
     return y.cpu().numpy()
 
 
+_CASE_WEIGHTS = {}
+
+
 def _case(oracle, n_out, k_in, gs, m_rows, seed, with_bias):
-    w = normal_weight(n_out, k_in, seed)
-    packed, scale, bias = group_quantize_compress_numpy(w, gs)
+    key = (n_out, k_in, gs, seed)  # (large weights take seconds to compress and decompress on the host: once per session)
+    if key not in _CASE_WEIGHTS:
+        packed, scale, bias = group_quantize_compress_numpy(normal_weight(n_out, k_in, seed), gs)
+        _CASE_WEIGHTS[key] = (packed, scale, bias, oracle.np_decompress(packed, scale, bias))
+    packed, scale, bias, w_dec = _CASE_WEIGHTS[key]
     x = activations(m_rows, k_in, seed + 1)
     out_bias = np.random.default_rng(seed + 2).normal(0, 1, (n_out,)).astype(np.float16) if with_bias else None
-    w_dec = oracle.np_decompress(packed, scale, bias)
     y_ref = oracle.np_linear(x, w_dec, out_bias)
     return x, packed, scale, bias, out_bias, y_ref
 
 
-@pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (16384, 4096), (4096, 16384)])
+@pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (16384, 4096), (4096, 16384), (20480, 4096), (12288, 4096)])
 @pytest.mark.parametrize("m_rows", [1, 2, 3, 4, 8, 16])
 def test_gemv_benchmark_shapes(hip, device, oracle, n_out, k_in, m_rows):
-    """Benchmark configurations 3 and 5: decode batches on the layer shapes of the 6B stack."""
+    """Benchmark configurations 3 and 5: decode batches on the layer shapes of the 6B stack, on a weight
+    large enough for the single call to go through the persistent kernel at up to four rows
+    (20480 x 4096) and on one whose row blocks do not divide evenly over the compute units (12288 x 4096)."""
     for with_bias in (False, True):
         x, packed, scale, bias, ob, y_ref = _case(oracle, n_out, k_in, 64, m_rows, 7, with_bias)
         y = _call(hip, "gq_gemv_f16", x, packed, scale, bias, ob, n_out, k_in, 64, device)
