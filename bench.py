@@ -421,19 +421,24 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     # contiguous).  Three entries per layer, 84 per pass, the same weight bytes; every entry reads
     # what earlier entries wrote, and the step to the next layer waits for all of the layer.
     joint = None
+    h0_joint = h0 * 100.0
     if m_rows == 1 and (modes is None or "sequence_decoder_data_flow_joint_output_streaming_layout" in modes):
         joint = {"w": [], "plain": None, "y": [torch.empty((1, hidden), dtype=torch.float16, device=device) for _ in range(2)],
                  "both": torch.empty((1, ffn + 3 * hidden), dtype=torch.float16, device=device)}
         for layer in range(n_layers):
             q, k, v, o, up, down = (mats[layer * 6 + role][2:] for role in range(6))
             vqk = tuple(torch.cat([v[part], q[part], k[part]], dim=0).contiguous() for part in range(3))
-            out = tuple(torch.cat([down[part], o[part]], dim=1).contiguous() for part in range(3))
+            out = [torch.cat([down[part], o[part]], dim=1).contiguous() for part in range(3)]
+            # without normalisation layers the joint product would multiply the layer input by 3.7 per layer
+            # (the four-entry schedule: by 1.6) and overflow fp16 after a dozen layers: scale the weight, i.e.
+            # its scales and biases, by 0.27
+            out = (out[0], (out[1].float() * 0.27).to(torch.float16), (out[2].float() * 0.27).to(torch.float16))
             joint["w"].append((prepacked[layer][2], hip.prepack_gemv(*vqk), hip.prepack_gemv(*out)))
             if layer == n_layers - 1:
                 joint["plain"] = (up, vqk, out)
 
     def data_flow_joint_output(seq):
-        h, last = h0, None
+        h, last = h0_joint, None
         for layer in range(n_layers):
             w_up, w_vqk, w_out = joint["w"][layer]
             seq.add(h, w_up, None, None, joint["both"][:, :ffn], None, wait_for=last)
@@ -467,6 +472,12 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         # the timed passes computed something: what the buffers hold now (the last layer's outputs)
         # equals single-call GEMVs on the same weights and the inputs the device had
         worst = 0.0
+
+        def worse(so_far, y, ref):
+            # (a result that is not finite, or a reference that is all zero, makes the error NaN, and NaN stays)
+            err = ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item()
+            return err if not (err <= so_far) else so_far
+
         last = (n_layers - 1) * 6
         if "joint_output" in mode:
             both, h_last = joint["both"], joint["y"][(n_layers - 2) % 2]
@@ -478,7 +489,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                 hip.call("gq_gemv_f16", x_in.data_ptr(), 1, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
                          y.shape[1], x_in.shape[1], GROUP, stream_handle())
                 torch.cuda.synchronize()
-                worst = max(worst, ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item())
+                worst = worse(worst, y, ref)
         elif "data_flow" in mode:
             h_last = y_o2[(n_layers - 2) % 2]
             checks = ((3, v_rows(y_qkv), y_o2[(n_layers - 1) % 2]), (4, h_last, ys[4]), (5, ys[4], ys[5]))
@@ -490,7 +501,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             hip.call("gq_gemv_f16", x_in.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
                      n_out, k_in, GROUP, stream_handle())
             torch.cuda.synchronize()
-            worst = max(worst, ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item())
+            worst = worse(worst, y, ref)
         results[mode]["max_error_vs_single_call"] = worst
         if not worst <= 2e-3 or results[mode]["status"] != 0:
             raise SystemExit(f"bench.py: stack mode {mode} (m={m_rows}) is wrong: error {worst}, status {results[mode]['status']}")
