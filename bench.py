@@ -80,6 +80,23 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def run_until_steady(fn, seconds=0.03):
+    """Untimed launches of fn(i) for `seconds`.  The first launches after a pause (here: after the
+    operands were made) run slower than the steady state -- the fused GEMV on 16384x4096 at batch 8:
+    14.0, 13.4, 13.0, 12.0 us over the first four blocks of 200 launches, 11.8 us from then on; the
+    packer on 4096x16384: 31.7, 32.8, 31.7, 31.4, 30.9, 30.8 us over the first six blocks of 100,
+    30.3 - 30.5 us from the eighth on.  Used by the benchmarks under `extra`; the headline decompress
+    figure is timed after exactly --warmup launches."""
+    import torch
+
+    t0, i0 = time.time(), 0
+    while time.time() - t0 < seconds:
+        for i in range(100):
+            fn(i0 + i)
+        i0 += 100
+        torch.cuda.synchronize()
+
+
 def make_weight(n_rows, n_cols, seed, outliers, device):
     """fp16 weight ~N(0, 0.02) (+ 0.1 % outliers at +-0.16), generated on the device from a seed."""
     import torch
@@ -147,6 +164,7 @@ def bench_compress(hip, device, steps, warmup, n_sets=4, rows=4096, cols=16384, 
         hip.call("gq_compress_f32" if f32 else "gq_compress_f16", w.data_ptr(), p.data_ptr(), s.data_ptr(), b.data_ptr(),
                  flag.data_ptr(), rows, cols // GROUP, GROUP, stream)
 
+    run_until_steady(step)
     ms = time_launches(step, steps, warmup)
     nbytes = rows * cols * ((4.0 if f32 else 2.0) + 0.5 + 4.0 / GROUP)
     return {"rows": rows, "cols": cols, "input": "float32" if f32 else "float16", "us": ms * 1e3, "bytes": nbytes,
@@ -251,15 +269,7 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
         else:
             hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP, stream)
 
-    # The first launches after a pause (here: after the weights were made) run slower than the steady
-    # state -- 16384x4096 at batch 8: 14.0, 13.4, 13.0, 12.0 us over the first four blocks of 200
-    # launches, 11.8 us from then on -- so launches are untimed until 30 ms of them have run.
-    t0, i0 = time.time(), 0
-    while time.time() - t0 < 0.03:
-        for i in range(100):
-            step(i0 + i)
-        i0 += 100
-        torch.cuda.synchronize()
+    run_until_steady(step)
     ms = time_launches(step, steps, warmup)
     w_bytes = n_out * k_in * (0.5 + 4.0 / GROUP)
     flops = 2.0 * m_rows * n_out * k_in
@@ -576,6 +586,7 @@ def main():
             hip.call("gq_decompress_f16_transposed", p.data_ptr(), s.data_ptr(), b.data_ptr(), outs_t[i % len(outs_t)].data_ptr(),
                      4096, 256, 16, stream_handle())
 
+        run_until_steady(step_t)
         ms_t = time_launches(step_t, 100, 10)
         extra["decompress_transposed"] = {"rows": 4096, "cols": 16384, "us": ms_t * 1e3, "gbs": dec["bytes"] / ms_t / 1e6,
                                           "hbm_frac": dec["bytes"] / ms_t / 1e6 / HBM_PEAK_GBS,
