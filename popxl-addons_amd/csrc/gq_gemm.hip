@@ -454,7 +454,15 @@ __device__ __forceinline__ void gemm_pipe2_body(
     }
 #pragma unroll
     for (int i = 0; i < FM; ++i) asm volatile("" : : "v"(a[1][i]));
-    if (FM == 2) {  // no MFMA group left to hide the expansion behind
+    if (FM == 1) {  // (the weight reads are older than the one fragment read issued since)
+#pragma unroll
+      for (int f = 0; f < FN; ++f) {
+        asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
+        s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
+        z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+      }
+    }
+    if (FM <= 2) {  // no MFMA group left to hide the expansion behind
 #pragma unroll
       for (int f = 0; f < FN; ++f) dequant_piece<1>(0, wq_next[f][0], s2n[f], z2n[f], st[f]);
     }
@@ -579,7 +587,7 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
   // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
   if ((k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    // Three tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
+    // Four tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
     // launch is as slow as its busiest compute unit: expected time = tiles per compute unit (256 of
     // them; a last, partly filled round runs faster: fewer workgroups share memory and clocks) x
     // time per tile, from measured times per 1024 input features with every compute unit busy:
@@ -596,6 +604,11 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
       return ((double)full + (rest ? 0.7 + 0.3 * (double)rest / 256.0 : 0.0)) * us_per_1024 * (double)k_in / 1024.0;
     };
     const double t_small = expected(128, 64, 8.0), t_mid = expected(256, 128, 22.0), t_large = expected(256, 256, 34.0);
+    // 64 x 64 (two groups of four waves of 32 x 32 that split K): 6.3 us per 1024 input features; for the
+    // batches and widths that leave the 128 x 64 tiles on half of the compute units or fewer (4096 x 4096
+    // at 256 rows: 26 against 31 us; 16384 x 4096 at 64 rows: 29 against 37 us)
+    const double t_tiny = k_in % 256 == 0 ? expected(64, 64, 6.3) : 1e30;
+    if (t_tiny < t_small && t_tiny < t_mid && t_tiny < t_large) return GQ_PIPE2(2, 2, 1, 1, 3, 2, 2);
     if (t_large <= t_mid && t_large <= t_small) return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
     if (t_mid <= t_small) return GQ_PIPE2(1, 4, 8, 1, 3, 1);                        // 256 x 128, 4 waves of 256 x 32
     // 128 x 64 (a workgroup on every compute unit at n_out = 16384), 4 waves of 64 x 32; two such

@@ -4,6 +4,8 @@
 // -- LinearGQ.build with dim=0 (popxl_addons/layers/linear_gq.py:99-109) without ever
 // writing the fp16 weight to memory.  HBM-bound on the packed weight: 0.5 + 4/gs bytes per
 // weight element.
+#include <algorithm>
+
 #include "gq_common.h"
 #include "gq_gemv_dequant.h"
 
@@ -353,8 +355,10 @@ bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packe
   const int64_t passes = (m_rows + 15) / 16;
   const double weights_mi = (double)n_out * (double)k_in / 1048576.0;
   const double t_pass = 4.7 + 0.124 * weights_mi * (k_in >= 8192 ? 1.35 : 1.0);
-  const int64_t tiles = (n_out + 63) / 64;
-  const double t_gemm = 7.5 * ((double)k_in / 1024.0) * (double)((tiles + 255) / 256);
+  const int64_t tiles = (n_out + 63) / 64, tiles64 = tiles * ((m_rows + 63) / 64);
+  double t_gemm = 7.5 * ((double)k_in / 1024.0) * (double)((tiles + 255) / 256);
+  // (the GEMM kernel's 64 x 64 tiles, where it has them: 7 per 1024 input features and round of 256)
+  if (k_in % 256 == 0) t_gemm = std::min(t_gemm, 7.0 * ((double)k_in / 1024.0) * (double)((tiles64 + 255) / 256));
   if ((double)passes * t_pass >= t_gemm) return false;
   for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
     const int64_t m = m_rows - m0 < 16 ? m_rows - m0 : 16;
