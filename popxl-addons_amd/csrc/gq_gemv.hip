@@ -32,11 +32,11 @@ namespace {
 // GS    64 or 128: scale/bias of a chunk are fetched as one 16/8-byte load per row and the lane's
 //       value is picked with a byte permute; 0: any power-of-two group >= 32, 2-byte loads.
 // FULL  k_in is a multiple of 512 (no slot predication).
-// XM    0: the lanes of batch row m fetch that row's x themselves, 16 bytes at a time (sixteen load
-//       instructions per chunk with 4 m_rows lanes active).  > 0 (m_rows <= XM, FULL): a chunk of a
-//       batch row is 1 KiB, fetched by ONE instruction of the whole wave and handed to the row's four
-//       lanes through LDS.  Measured on 4096 x 4096: the x loads of XM = 0 cost 0.8 us of 5.9 at one
-//       batch row and 1.9 us of 7.1 at eight.
+// XM    1, 4, 8 or 16 >= m_rows: the 1 KiB of x that a chunk needs of a batch row is fetched by ONE load
+//       instruction of the whole wave, ahead of the weight loads, and handed to the row's four lanes
+//       through LDS.  (Those four lanes fetching their sixteen 16-byte pieces themselves -- sixteen
+//       load instructions per chunk with 4 m_rows lanes active -- cost 0.8 us of 5.9 at one batch row
+//       and 1.9 us of 7.1 at eight on 4096 x 4096.)
 constexpr int gemv_region_bytes(int r, int xm) { return (xm > r ? xm : r) * 1024; }
 
 template <int NWAVES, int R, int GS, bool FULL, int XM>
@@ -44,7 +44,6 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
     int gs_shift, int act) {
-  static_assert(XM == 0 || FULL, "staged x needs whole chunks");
   // per wave: the x chunk of up to XM batch rows while the wave walks K, its partial sums at the end
   constexpr int kRegion = gemv_region_bytes(R, XM);
   extern __shared__ __attribute__((aligned(16))) char region_base[];
@@ -54,8 +53,6 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
   const int n_slots = k_in >> 7;
   const int n_chunks = (n_slots + 3) >> 2;
   const int groups_per_row = k_in >> gs_shift;
-  const bool has_x = r < m_rows;
-  const half_t *xrow = x + (int64_t)(has_x ? r : 0) * k_in + kc * 32;
   const uint4_t *wrow[R];
   const half_t *srow[R], *brow[R];
 #pragma unroll
@@ -76,14 +73,15 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
   // staged x: 16-byte piece p of batch row m lies at piece p ^ m of the row's KiB, so that the sixteen
   // rows read by lanes of one slice fall on different banks
   char *const stage = region[wave];
-  const int x_row = has_x ? r : 0;  // (columns past the batch are never stored: they may hold any row)
+  const int x_row = r < m_rows ? r : 0;  // (columns past the batch are never stored: they may hold any row)
   for (int c = wave; c < n_chunks; c += NWAVES) {
-    uint4_t xq[XM > 0 ? XM : 1];
-    if constexpr (XM > 0) {
+    uint4_t xq[XM];
+    {
 #pragma unroll
       for (int m = 0; m < XM; ++m) {
         xq[m] = uint4_t{0u, 0u, 0u, 0u};
-        if (m < m_rows) xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + c * 512 + lane * 8);
+        if (m < m_rows && (FULL || c * 512 + lane * 8 < k_in))  // (k_in is a multiple of 128: a piece is whole or absent)
+          xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + c * 512 + lane * 8);
       }
     }
     uint4_t wq[R][4];
@@ -134,20 +132,14 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     half8_t xp[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int slot = c * 4 + j;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        uint4_t q = {0u, 0u, 0u, 0u};
-        if constexpr (XM > 0) {
-          if (j == 0 && s == 0) {
+        if (j == 0 && s == 0) {
 #pragma unroll
-            for (int m = 0; m < XM; ++m)
-              if (m < m_rows) *reinterpret_cast<uint4_t *>(stage + m * 1024 + ((lane ^ m) & 63) * 16) = xq[m];
-          }
-          q = *reinterpret_cast<const uint4_t *>(stage + x_row * 1024 + ((j * 16 + kc * 4 + s) ^ x_row) * 16);
-        } else {
-          if (has_x && (FULL || slot < n_slots)) q = *reinterpret_cast<const uint4_t *>(xrow + slot * 128 + s * 8);
+          for (int m = 0; m < XM; ++m)
+            if (m < m_rows) *reinterpret_cast<uint4_t *>(stage + m * 1024 + ((lane ^ m) & 63) * 16) = xq[m];
         }
+        const uint4_t q = *reinterpret_cast<const uint4_t *>(stage + x_row * 1024 + ((j * 16 + kc * 4 + s) ^ x_row) * 16);
         xp[j][s] = permute_x(q);
       }
     }
@@ -311,20 +303,20 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL, XM);   \
     else GQ_GEMV_LAUNCH(NW, 1, GS, FULL, XM);               \
   } while (0)
-    // whole chunks: x through LDS, one load instruction per batch row and chunk (the rows of x are
-    // 16-byte aligned then), on eight waves whatever the length of the rows (measured on 4096 x 16384:
+    // x through LDS, one load instruction per batch row and chunk (the rows of x are 16-byte aligned:
+    // k_in % 128 == 0), on eight waves whatever the length of the rows (measured on 4096 x 16384:
     // 16 waves are no faster with x staged; without, eight rows took 20.1 us against 14.7 us)
-#define GQ_GEMV_BY_M(GS)                                    \
+#define GQ_GEMV_BY_M(GS, FULL)                              \
   do {                                                      \
-    if (m_rows == 1) GQ_GEMV_BY_R(8, GS, true, 1);          \
-    else if (m_rows <= 4) GQ_GEMV_BY_R(8, GS, true, 4);     \
-    else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, true, 8);     \
-    else GQ_GEMV_BY_R(8, GS, true, 16);                     \
+    if (m_rows == 1) GQ_GEMV_BY_R(8, GS, FULL, 1);          \
+    else if (m_rows <= 4) GQ_GEMV_BY_R(8, GS, FULL, 4);     \
+    else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, FULL, 8);     \
+    else GQ_GEMV_BY_R(8, GS, FULL, 16);                     \
   } while (0)
-    if (gs_mode == 64) GQ_GEMV_BY_M(64);
-    else if (gs_mode == 128) GQ_GEMV_BY_M(128);
-    else if (full) GQ_GEMV_BY_M(0);
-    else GQ_GEMV_BY_R(8, 0, false, 0);
+    if (gs_mode == 64) GQ_GEMV_BY_M(64, true);
+    else if (gs_mode == 128) GQ_GEMV_BY_M(128, true);
+    else if (full) GQ_GEMV_BY_M(0, true);
+    else GQ_GEMV_BY_M(0, false);  // (a last chunk of 128, 256 or 384 features, e.g. k_in = 11008)
 #undef GQ_GEMV_BY_M
 #undef GQ_GEMV_BY_R
 #undef GQ_GEMV_LAUNCH

@@ -91,6 +91,9 @@ def test_gemv_benchmark_shapes(hip, device, oracle, n_out, k_in, m_rows):
         (16400, 512, 64, 16),
         (100, 8192, 64, 2),  # several chunks per wave
         (100, 8192, 64, 11),
+        (300, 11008, 64, 5),  # a last chunk of 256 features (21 whole chunks before it)
+        (64, 896, 64, 16),
+        (8200, 640, 64, 1),
         # the same with groups of 128 (8-byte scale / bias loads) and of 32 and 256 (2-byte loads)
         (48, 1024, 128, 5),
         (8200, 512, 128, 2),
