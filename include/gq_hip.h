@@ -180,7 +180,9 @@ int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16
  * sequence have completed (0 <= wait_entries <= i; 0 = no dependency, i = every earlier entry).
  * Set it past the entry that produces x or out_bias of entry i.  Entries may otherwise overlap
  * and complete in any order: an entry that overwrites memory which an earlier entry reads or
- * writes must wait for that entry as well.
+ * writes must wait for that entry as well.  The x of an entry may be (part of) the y of one earlier
+ * entry or, at one batch row, of several earlier entries whose y lie end to end in memory (two
+ * projections whose results are added, as one entry over the concatenation of their inputs).
  *
  * For group_size 64, k_in % 512 == 0, m_rows <= 4 and 16-byte aligned pointers the whole sequence
  * runs as one persistent kernel (one workgroup per compute unit) that streams the packed weights
