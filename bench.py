@@ -284,6 +284,7 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
 
 
 FLOW_KERNEL_MODES = ("sequence_decoder_data_flow_streaming_layout", "sequence_decoder_data_flow_joint_output_streaming_layout",
+                     "sequence_decoder_data_flow_two_entries_streaming_layout",
                      "sequence_no_waits_streaming_layout")
 
 
@@ -432,7 +433,10 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     # what earlier entries wrote, and the step to the next layer waits for all of the layer.
     joint = None
     h0_joint = h0 * 100.0
-    if m_rows == 1 and (modes is None or "sequence_decoder_data_flow_joint_output_streaming_layout" in modes):
+    # ... and with up, v, q and k, which all read the layer input, stacked into one 28672-row entry
+    # (LinearGQ.fuse) in front of it: two entries per layer, 56 per pass.
+    joint_modes = ("sequence_decoder_data_flow_joint_output_streaming_layout", "sequence_decoder_data_flow_two_entries_streaming_layout")
+    if m_rows == 1 and (modes is None or any(mode in modes for mode in joint_modes)):
         joint = {"w": [], "plain": None, "y": [torch.empty((1, hidden), dtype=torch.float16, device=device) for _ in range(2)],
                  "both": torch.empty((1, ffn + 3 * hidden), dtype=torch.float16, device=device)}
         for layer in range(n_layers):
@@ -443,16 +447,25 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             # (the four-entry schedule: by 1.6) and overflow fp16 after a dozen layers: scale the weight, i.e.
             # its scales and biases, by 0.27
             out = (out[0], (out[1].float() * 0.27).to(torch.float16), (out[2].float() * 0.27).to(torch.float16))
-            joint["w"].append((prepacked[layer][2], hip.prepack_gemv(*vqk), hip.prepack_gemv(*out)))
+            first = tuple(torch.cat([up[part], vqk[part]], dim=0).contiguous() for part in range(3))
+            joint["w"].append((prepacked[layer][2], hip.prepack_gemv(*vqk), hip.prepack_gemv(*out), hip.prepack_gemv(*first)))
             if layer == n_layers - 1:
                 joint["plain"] = (up, vqk, out)
 
     def data_flow_joint_output(seq):
         h, last = h0_joint, None
         for layer in range(n_layers):
-            w_up, w_vqk, w_out = joint["w"][layer]
+            w_up, w_vqk, w_out, _ = joint["w"][layer]
             seq.add(h, w_up, None, None, joint["both"][:, :ffn], None, wait_for=last)
             a = seq.add(h, w_vqk, None, None, joint["both"][:, ffn:], None, wait_for=last)
+            h = joint["y"][layer % 2]
+            last = seq.add(joint["both"][:, : ffn + hidden], w_out, None, None, h, None, wait_for=a)
+
+    def data_flow_two_entries(seq):
+        h, last = h0_joint, None
+        for layer in range(n_layers):
+            *_, w_out, w_first = joint["w"][layer]
+            a = seq.add(h, w_first, None, None, joint["both"], None, wait_for=last)
             h = joint["y"][layer % 2]
             last = seq.add(joint["both"][:, : ffn + hidden], w_out, None, None, h, None, wait_for=a)
 
@@ -463,8 +476,9 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                        ("sequence_decoder_data_flow", lambda seq: data_flow(seq, streaming=False)),
                        ("sequence_decoder_data_flow_streaming_layout", data_flow),
                        ("sequence_decoder_data_flow_joint_output_streaming_layout", data_flow_joint_output),
+                       ("sequence_decoder_data_flow_two_entries_streaming_layout", data_flow_two_entries),
                        ("sequence_no_waits", free), ("sequence_no_waits_streaming_layout", free_streaming)):
-        if (modes is not None and mode not in modes) or ("joint_output" in mode and joint is None):
+        if (modes is not None and mode not in modes) or (mode in joint_modes and joint is None):
             continue
         seq = hip.GemvSequence(device)
         fill(seq)
@@ -489,7 +503,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             return err if not (err <= so_far) else so_far
 
         last = (n_layers - 1) * 6
-        if "joint_output" in mode:
+        if mode in joint_modes:  # (the stacked first entry computes what up and v|q|k compute separately)
             both, h_last = joint["both"], joint["y"][(n_layers - 2) % 2]
             singles = ((h_last, joint["plain"][0], both[:, :ffn]), (h_last, joint["plain"][1], both[:, ffn:]),
                        (both[:, : ffn + hidden], joint["plain"][2], joint["y"][(n_layers - 1) % 2]))

@@ -399,6 +399,34 @@ def test_gemv_sequence_x_from_several_producers(hip, device, oracle, streaming, 
             assert_close(yy, oracle.np_linear(x_in.cpu().numpy(), w_dec, None, activation), i)
 
 
+
+def test_gemv_sequence_two_entries_per_layer(hip, device, oracle):
+    """The decoder block as two entries: up, v, q and k stacked into one 28672 x 4096 entry (seven row
+    blocks per workgroup, passed on in parts of 2, 2, 2 and 1), then the joint output product over the
+    first 20480 of its results.  Two layers, streaming layout, batch 1; every entry against the oracle
+    applied to what the device fed it."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    hidden, ffn = 4096, 16384
+    seq, checks = GemvSequence(device), []
+    x = to_dev(activations(1, hidden, 4), device)
+    for layer in range(2):
+        first = torch.full((1, ffn + 3 * hidden), float("nan"), dtype=torch.float16, device=device)
+        y = torch.full((1, hidden), float("nan"), dtype=torch.float16, device=device)
+        for x_in, n_out, out, activation in ((x, ffn + 3 * hidden, first, "relu"), (first[:, : ffn + hidden], hidden, y, None)):
+            packed, scale, bias, w_dec = _full_size_weight(oracle, n_out, x_in.shape[1], 8000 + len(checks))
+            seq.add(x_in, prepack_gemv(*(to_dev(a, device) for a in (packed, scale, bias))), None, None, out, activation=activation)
+            checks.append((x_in, w_dec, out, activation))
+        x = y
+    for _ in range(3):
+        for _, _, out, _ in checks:
+            out.fill_(float("nan"))
+        seq.run()
+        torch.cuda.synchronize()
+        assert int(seq.status.item()) == 0
+        for i, (x_in, w_dec, out, activation) in enumerate(checks):
+            assert_close(out.cpu().numpy(), oracle.np_linear(x_in.cpu().numpy(), w_dec, None, activation), i)
+
 @pytest.mark.parametrize("m_rows,chained", [(1, False), (2, False), (4, False), (1, True), (4, True)])
 def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
     """Weights in the streaming layout of gq_gemv_prepack_f16 give what the same sequence gives on
