@@ -71,7 +71,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
   for (int i = 0; i < R; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   // staged x: 16-byte piece p of batch row m lies at piece p ^ m of the row's KiB, so that the sixteen
-  // rows read by lanes of one slice fall on different banks
+  // rows read by the lanes of one slice are spread over the banks (measured on 4096 x 4096: no
+  // bank-conflict cycles at one batch row, 2.5 per LDS instruction at eight -- 2 % of the waves' cycles)
   char *const stage = region[wave];
   const int x_row = r < m_rows ? r : 0;  // (columns past the batch are never stored: they may hold any row)
   for (int c = wave; c < n_chunks; c += NWAVES) {
