@@ -99,8 +99,17 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
           wq[i][j] = uint4_t{0u, 0u, 0u, 0u};
       }
       if constexpr (GS == 64) {
-        const uint4_t sv = *reinterpret_cast<const uint4_t *>(srow[i] + c * 8);
-        const uint4_t bv = *reinterpret_cast<const uint4_t *>(brow[i] + c * 8);
+        // A last chunk of fewer than four slots: the 16 bytes END with the row (the launcher sees to it
+        // that there is a whole chunk in front), and the dword of slot j is found `back` places later.
+        // The dwords that then stand for the absent slots belong to earlier groups of the row: finite
+        // numbers, multiplied by codes and x that are zero.
+        const int back = (!FULL && c == n_chunks - 1) ? 4 - (n_slots - c * 4) : 0;
+        uint4_t sv = *reinterpret_cast<const uint4_t *>(srow[i] + c * 8 - back * 2);
+        uint4_t bv = *reinterpret_cast<const uint4_t *>(brow[i] + c * 8 - back * 2);
+        if (!FULL) {
+          if (back & 1) sv = uint4_t{sv.y, sv.z, sv.w, sv.x}, bv = uint4_t{bv.y, bv.z, bv.w, bv.x};
+          if (back & 2) sv = uint4_t{sv.z, sv.w, sv.x, sv.y}, bv = uint4_t{bv.z, bv.w, bv.x, bv.y};
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           s2[i][j] = __builtin_amdgcn_perm(sv[j], sv[j], half_sel);
@@ -271,7 +280,9 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     // the GS == 64 / 128 instantiations fetch a chunk's scales and biases as one 16 / 8-byte load per
     // row: that needs the arrays aligned accordingly; otherwise the 2-byte loads of GS == 0 serve
     const uintptr_t sb_align = (uintptr_t)scale | (uintptr_t)bias;
-    const int gs_mode = (group_size == 64 && full && sb_align % 16 == 0)
+    // (group 64 with a partial last chunk, e.g. k_in = 11008: the rows of scale / bias are then only
+    // 4-byte aligned, which the 16-byte loads take, and the last load reaches back into the chunk before)
+    const int gs_mode = (group_size == 64 && (full || k_in > 512) && sb_align % 16 == 0)
                             ? 64
                             : ((group_size == 128 && full && sb_align % 8 == 0) ? 128 : 0);
     const unsigned blocks = (unsigned)((row_blocks + r - 1) / r);
@@ -314,7 +325,8 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, FULL, 8);     \
     else GQ_GEMV_BY_R(8, GS, FULL, 16);                     \
   } while (0)
-    if (gs_mode == 64) GQ_GEMV_BY_M(64, true);
+    if (gs_mode == 64 && full) GQ_GEMV_BY_M(64, true);
+    else if (gs_mode == 64) GQ_GEMV_BY_M(64, false);
     else if (gs_mode == 128) GQ_GEMV_BY_M(128, true);
     else if (full) GQ_GEMV_BY_M(0, true);
     else GQ_GEMV_BY_M(0, false);  // (a last chunk of 128, 256 or 384 features, e.g. k_in = 11008)
