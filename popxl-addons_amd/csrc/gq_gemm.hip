@@ -593,7 +593,7 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     // time per tile, from measured times per 1024 input features with every compute unit busy:
     //   128 x 64   8 us   (16384 x 4096 at 128 rows: 34.5 us)
     //   256 x 128  22 us  (16384 x 4096 at 512 rows: 87 us; 16 us with an eighth of the compute units busy)
-    //   256 x 256  34 us  (two per compute unit at a time; 16384 x 4096 at 2048 rows: 271 us, at 1024 rows 140 us)
+    //   256 x 256  34 us  (16384 x 4096 at 2048 rows: two rounds, 271 us; at 1024 rows one, 140 us)
     // Fixed thresholds on the batch alone (256 x 128 from 256 rows, 256 x 256 from 1024) left weights
     // with 4096 outputs on 16 to 64 workgroups: 4096 x 4096 at 512 rows took 75.6 us, now 36 us.  With each
     // shape forced in turn, this choice was the fastest or within 2 % of it for five weight shapes
