@@ -646,6 +646,17 @@ def main():
             extra["gemm"].append(r)
             log(f"  gemm m={m} [16384x4096]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
             torch.cuda.empty_cache()
+        # the stack's other layer shapes (4096 outputs: few tiles, where the choice of tile matters most) and the
+        # batches between the GEMV's 16 rows and full GEMM tiles, through the entry that the layer calls
+        extra["gemm_other_shapes"] = []
+        for entry, m, n_out, k_in in (("gq_gemm_f16", 512, 4096, 4096), ("gq_gemm_f16", 512, 4096, 16384),
+                                      ("gq_linear_f16", 32, 4096, 4096), ("gq_linear_f16", 64, 16384, 4096)):
+            r = bench_linear(hip, device, entry, m, n_out, k_in, 30, 5, n_sets=4,
+                             kernel="gemm_pipe2_kernel" if entry == "gq_gemm_f16" else "gemv_mfma_kernel passes / gemm_pipe2_kernel")
+            r["entry"] = entry
+            extra["gemm_other_shapes"].append(r)
+            log(f"  {entry} m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s")
+            torch.cuda.empty_cache()
     if args.only in ("stack", "all"):
         extra["stack"] = []
         modes = tuple(m for m in args.stack_modes.split(",") if m) or None
