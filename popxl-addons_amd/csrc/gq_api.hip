@@ -183,7 +183,11 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                                       group_size, activation);
   if (rc <= 0) return rc;
   const int64_t need = gq::linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
-  if (need > 0) {
+  // (more than 16 rows: the workspace is an option -- with one that is large enough the batch may run as
+  // passes of the decode kernel, without it the prefill kernel runs)
+  if (m_rows > 16 && (!workspace || workspace_bytes < need || gq::misaligned(workspace, 16))) {
+    workspace = nullptr;
+  } else if (need > 0) {
     if (!workspace) return gq::fail(GQ_ERR_NULL_POINTER, "gq_linear_kn_act_f16: this problem needs a workspace of %lld bytes",
                                     (long long)need);
     if (gq::misaligned(workspace, 16))

@@ -367,10 +367,28 @@ bool kn_fast_shape(const uint16_t *x, const uint16_t *packed, int64_t n_out, int
 
 }  // namespace
 
+// Batches of 17 to 128 rows as passes of the decode kernel over 16 rows each, against the prefill
+// kernel, whose 128 x 128 tiles are mostly empty there and few when n_out is small.  From measured
+// times (us): a pass of 16 rows 18 + 0.37 per Mi weights (23.9 on 4096 -> 4096, 41.8 on
+// 4096 -> 16384, 41.3 on 16384 -> 4096), fewer rows in the last pass less; the prefill kernel 1.4 per
+// 64 input features and round of 256 tiles (84 / 103 / 370 on the same shapes, whatever the batch up to
+// 128).  Measured: 16384 -> 4096 at 32 rows 87 against 367, 4096 -> 4096 at 32 rows 49 against 83.
+bool kn_passes_faster(int64_t m_rows, int64_t n_out, int64_t k_in) {
+  if (m_rows <= 16 || m_rows > 128) return false;
+  const double t16 = 18.0 + 0.37 * (double)n_out * (double)k_in / 1048576.0;
+  const int64_t rest = m_rows % 16;
+  const double last = rest == 0 ? 0.0 : (rest <= 2 ? 0.45 : (rest <= 4 ? 0.55 : (rest <= 8 ? 0.7 : 1.0)));
+  const double t_passes = ((double)(m_rows / 16) + last) * t16;
+  const int64_t tiles = (n_out + BN - 1) / BN;  // (one row of tiles up to 128 rows)
+  const double t_prefill = 1.4 * (double)k_in / 64.0 * (double)((tiles + 255) / 256);
+  return t_passes < t_prefill;
+}
+
 // Scratch bytes the decode kernel needs for this problem (0: none): the arrival counters (a fixed
 // 16 KiB at the start, so that calls of any shape find them at the same place), then 2 KiB of
 // fp32 partial sums per (K slab, strip, batch-row pair).
 int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (m_rows > 16 && kn_passes_faster(m_rows, n_out, k_in)) m_rows = 16;  // passes of the decode kernel over 16 rows
   if (m_rows < 1 || m_rows > 16 || k_in < 1) return 0;
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   if (!pow2 || group_size < 32 || n_out % 32 != 0 || n_out < 32 || n_out > (int64_t)kMaxStrips * kStrip) return 0;
@@ -391,6 +409,16 @@ int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
   half_t *yh = reinterpret_cast<half_t *>(y);
   const bool fast = kn_fast_shape(x, packed, n_out, k_in, group_size);
   const int gs_shift = fast ? __builtin_ctzll((unsigned long long)group_size) : 0;
+  if (fast && m_rows > 16 && kn_passes_faster(m_rows, n_out, k_in) &&
+      (workspace || linear_kn_workspace_bytes(16, n_out, k_in, group_size) == 0)) {
+    for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
+      const int64_t m = m_rows - m0 < 16 ? m_rows - m0 : 16;
+      const int rc = launch_linear_kn(x + m0 * k_in, m, packed, scale, bias, out_bias, y + m0 * n_out, n_out, k_in, group_size,
+                                      act, workspace, stream);
+      if (rc != GQ_OK) return rc;
+    }
+    return GQ_OK;
+  }
   if (fast && m_rows <= 16) {
     int64_t slab = 0;
     const int splits = kn_splits(m_rows, n_out, k_in, &slab);
@@ -438,7 +466,8 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 int launch_linear_kn_noalloc(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                              const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                              int64_t group_size, int act, hipStream_t stream) {
-  const int64_t need = linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
+  int64_t need = linear_kn_workspace_bytes(m_rows, n_out, k_in, group_size);
+  if (need > kScratchBytes && m_rows > 16) need = 0;  // (no passes of the decode kernel then: the prefill kernel needs no scratch)
   if (need > kScratchBytes)
     return fail(GQ_ERR_UNSUPPORTED,
                 "gq_linear_kn_act_noalloc_f16: m_rows=%lld n_out=%lld k_in=%lld needs %lld bytes of scratch, the built-in "
