@@ -164,9 +164,12 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
  * counterpart in the reference.  The partial sums and arrival counters live in a device array
  * inside the library (one copy per GPU, 16 KiB + GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES, held until the
  * process ends); the call allocates and frees nothing.  Same arguments, results bit for bit those
- * of gq_linear_kn_act_f16.  A problem whose gq_linear_kn_workspace_bytes() exceeds that size is
- * rejected with GQ_ERR_UNSUPPORTED (every problem of up to 8 rows fits; of the 6B layer shapes,
- * 4096 and 16384 outputs fit up to 16 rows, the fused 12288-wide projection up to 8).
+ * of gq_linear_kn_act_f16.  A problem of up to 16 rows whose gq_linear_kn_workspace_bytes() exceeds
+ * that size is rejected with GQ_ERR_UNSUPPORTED (every problem of up to 8 rows fits; of the 6B layer
+ * shapes, 4096 and 16384 outputs fit up to 16 rows, the fused 12288-wide projection up to 8).  Above
+ * 16 rows nothing is rejected: where the 16-row passes that gq_linear_kn_act_f16 would run do not
+ * fit, the prefill kernel, which needs no scratch, runs (the same result to the tolerance of the
+ * fused paths, not bit for bit).
  * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race.
  */
 #define GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES (4 << 20)
