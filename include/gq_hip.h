@@ -147,10 +147,13 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
  * for the same sizes (0: none needed, workspace may be NULL).  Its first 16 KiB hold arrival
  * counters: the caller zeroes them once, every call leaves them zero, so one workspace serves
  * calls of any shape -- one at a time: calls that share a workspace must not overlap.
- * For 17 <= m_rows <= 128 gq_linear_kn_workspace_bytes() returns the same figure as for 16 rows
- * where the batch is expected to run faster as passes of that kernel over 16 rows each (large
- * weights, above all narrow ones); there the workspace is an option: without it, or with one that
- * is too small, the prefill kernel runs and gives the same result.
+ * For m_rows > 16 the workspace is an option.  gq_linear_kn_workspace_bytes() is non-zero where the
+ * 128 x 128 output tiles are too few for the device (a weight with 4096 outputs has 32 per 128 rows):
+ * with the workspace the prefill kernel divides the input features over several workgroups per tile,
+ * whose binary32 partial sums meet there (or, for 17 to 128 rows, the batch runs as passes of the
+ * decode kernel over 16 rows each where those are expected to be faster); without it, or with one
+ * that is too small, the prefill kernel runs undivided and gives the same result to the tolerance
+ * of the fused paths.
  */
 int64_t gq_linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
 int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,

@@ -244,11 +244,16 @@ constexpr int BM = 128, BN = 128, BK = 64, LDK = BK + 8;
 
 __device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
+// gridDim.z > 1: the workgroups of a tile divide K into slabs of `slab` input features; their fp32
+// accumulators meet in `partial` ([slab][tile][element][thread], a float4 per element quarter) and the
+// last one to arrive at the tile (arrival counters as in the decode kernel: zero before and after)
+// adds them in the order of the slabs and stores y.
 __global__ __launch_bounds__(256) void gemm_kn_tile_kernel(const half_t *__restrict__ x, int m_rows,
                                                            const char *__restrict__ packed, const half_t *__restrict__ scale,
                                                            const half_t *__restrict__ bias,
                                                            const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                           int n_out, int k_in, int gs_shift, int act) {
+                                                           int n_out, int k_in, int gs_shift, int act, int slab,
+                                                           float4_t *__restrict__ partial, unsigned *__restrict__ counters) {
   __shared__ __attribute__((aligned(16))) half_t As[BM][LDK];
   __shared__ __attribute__((aligned(16))) half_t Bs[BN][LDK];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -300,12 +305,13 @@ __global__ __launch_bounds__(256) void gemm_kn_tile_kernel(const half_t *__restr
   };
 
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
-  load_tile(0);
-  for (int k0 = 0; k0 < k_in; k0 += BK) {
+  const int k_begin = (int)blockIdx.z * slab, k_end = min(k_in, k_begin + slab);
+  load_tile(k_begin);
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
     __syncthreads();
     store_tile();
     __syncthreads();
-    if (k0 + BK < k_in) load_tile(k0 + BK);
+    if (k0 + BK < k_end) load_tile(k0 + BK);
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
       half8_t a[2], b[2];
@@ -319,6 +325,50 @@ __global__ __launch_bounds__(256) void gemm_kn_tile_kernel(const half_t *__restr
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  if (gridDim.z > 1) {
+    __shared__ unsigned tile_arrived;
+    const int n_splits = gridDim.z, tile = blockIdx.y * gridDim.x + blockIdx.x, n_tiles = gridDim.x * gridDim.y;
+    float4_t *mine = partial + ((int64_t)blockIdx.z * n_tiles + tile) * (16 * 256) + tid;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4)
+          store_coherent(mine + ((i * 2 + j) * 4 + q4) * 256,
+                         float4_t{acc[i][j][4 * q4], acc[i][j][4 * q4 + 1], acc[i][j][4 * q4 + 2], acc[i][j][4 * q4 + 3]});
+    // the workgroup's partial sums are in memory before it counts itself in
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned before = __hip_atomic_fetch_add(counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      tile_arrived = before;
+      if (before == (unsigned)n_splits - 1)  // the last one: leave the counter at zero for the next launch
+        __hip_atomic_store(counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (tile_arrived != (unsigned)n_splits - 1) return;
+    // the slabs in order (the same result whoever arrives last), a slab's sixteen loads in flight at a time
+    const float4_t *first = partial + (int64_t)tile * (16 * 256) + tid;
+    const int64_t stride = (int64_t)n_tiles * (16 * 256);  // float4 between consecutive slabs
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+      float4_t v[16];
+      load_coherent<16>(first + sp * stride, 256, v);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] += v[(i * 2 + j) * 4 + (e >> 2)][e & 3];
     }
   }
 
@@ -368,19 +418,24 @@ bool kn_fast_shape(const uint16_t *x, const uint16_t *packed, int64_t n_out, int
 }  // namespace
 
 // Batches of 17 to 128 rows as passes of the decode kernel over 16 rows each, against the prefill
-// kernel, whose 128 x 128 tiles are mostly empty there and few when n_out is small.  From measured
-// times (us): a pass of 16 rows 18 + 0.37 per Mi weights (23.9 on 4096 -> 4096, 41.8 on
-// 4096 -> 16384, 41.3 on 16384 -> 4096), fewer rows in the last pass less; the prefill kernel 1.4 per
-// 64 input features and round of 256 tiles (84 / 103 / 370 on the same shapes, whatever the batch up to
-// 128).  Measured: 16384 -> 4096 at 32 rows 87 against 367, 4096 -> 4096 at 32 rows 49 against 83.
+// kernel, whose 128 x 128 tiles are mostly empty there.  From measured times (us): a pass of 16 rows
+// 18 + 0.37 per Mi weights (23.9 on 4096 -> 4096, 41.8 on 4096 -> 16384, 41.3 on 16384 -> 4096), fewer
+// rows in the last pass less; the prefill kernel 1.4 per 64 input features of a slab and round of 256
+// workgroups, plus 10 for the partial sums where K is divided (measured with the workspace for that:
+// 25 - 28 / 61 - 63 / 61 - 64 on the same shapes, whatever the batch up to 128; undivided 84 / 103 / 370).
+// With K divided the prefill kernel wins nearly everywhere; the passes remain for weights whose slabs
+// cannot be short enough (few input features, many outputs).
 bool kn_passes_faster(int64_t m_rows, int64_t n_out, int64_t k_in) {
   if (m_rows <= 16 || m_rows > 128) return false;
   const double t16 = 18.0 + 0.37 * (double)n_out * (double)k_in / 1048576.0;
   const int64_t rest = m_rows % 16;
   const double last = rest == 0 ? 0.0 : (rest <= 2 ? 0.45 : (rest <= 4 ? 0.55 : (rest <= 8 ? 0.7 : 1.0)));
   const double t_passes = ((double)(m_rows / 16) + last) * t16;
-  const int64_t tiles = (n_out + BN - 1) / BN;  // (one row of tiles up to 128 rows)
-  const double t_prefill = 1.4 * (double)k_in / 64.0 * (double)((tiles + 255) / 256);
+  // (with K divided over workgroups: a slab's steps, and some 10 us for the partial sums to meet)
+  int64_t slab = 0;
+  const int splits = kn_prefill_splits(m_rows, n_out, k_in, &slab);
+  const int64_t tiles = (n_out + BN - 1) / BN * splits;  // (one row of tiles up to 128 rows)
+  const double t_prefill = 1.4 * (double)slab / 64.0 * (double)((tiles + 255) / 256) + (splits > 1 ? 10.0 : 0.0);
   return t_passes < t_prefill;
 }
 
@@ -389,6 +444,15 @@ bool kn_passes_faster(int64_t m_rows, int64_t n_out, int64_t k_in) {
 // fp32 partial sums per (K slab, strip, batch-row pair).
 int64_t linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
   if (m_rows > 16 && kn_passes_faster(m_rows, n_out, k_in)) m_rows = 16;  // passes of the decode kernel over 16 rows
+  if (m_rows > 16) {
+    // the prefill kernel with K divided over workgroups: counters, then 64 KiB of partial sums per (slab, tile)
+    if (!kn_prefill_shape(n_out, k_in, group_size)) return 0;
+    int64_t slab = 0;
+    const int splits = kn_prefill_splits(m_rows, n_out, k_in, &slab);
+    if (splits == 1) return 0;
+    const int64_t tiles = ((n_out + BN - 1) / BN) * ((m_rows + BM - 1) / BM);
+    return (int64_t)kMaxStrips * 4 + splits * tiles * 65536;
+  }
   if (m_rows < 1 || m_rows > 16 || k_in < 1) return 0;
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   if (!pow2 || group_size < 32 || n_out % 32 != 0 || n_out < 32 || n_out > (int64_t)kMaxStrips * kStrip) return 0;
@@ -440,8 +504,15 @@ int launch_linear_kn(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
   if (fast && k_in % BK == 0 && ((uintptr_t)x % 16) == 0) {
     const dim3 grid((unsigned)((n_out + BN - 1) / BN), (unsigned)((m_rows + BM - 1) / BM));
     if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_linear_kn: m_rows=%lld too large", (long long)m_rows);
-    gemm_kn_tile_kernel<<<grid, dim3(256), 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, oh,
-                                                        yh, (int)n_out, (int)k_in, gs_shift, act);
+    // K divided over workgroups where the tiles are few and the caller brought the workspace for it
+    int64_t slab = k_in;
+    int splits = workspace ? kn_prefill_splits(m_rows, n_out, k_in, &slab) : 1;
+    if (splits == 1) slab = k_in;
+    unsigned *counters = static_cast<unsigned *>(workspace);
+    float4_t *partial = workspace ? reinterpret_cast<float4_t *>(counters + kMaxStrips) : nullptr;
+    const dim3 grid3(grid.x, grid.y, (unsigned)splits);
+    gemm_kn_tile_kernel<<<grid3, dim3(256), 0, stream>>>(xh, (int)m_rows, reinterpret_cast<const char *>(packed), sh, bh, oh,
+                                                         yh, (int)n_out, (int)k_in, gs_shift, act, (int)slab, partial, counters);
     return check_launch("gemm_kn_tile_kernel");
   }
   const unsigned blocks = (unsigned)((n_out + 255) / 256);

@@ -63,11 +63,11 @@ def test_abi_version_and_error_text_without_gpu():
     assert need > 16384 and need <= 16384 + 64 * 16384 * 4 and need == lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 32)
     assert lib.gq_linear_kn_workspace_bytes(4, 16384, 4096, 64) == 16384 + (need - 16384) * 2  # two batch-row pairs
     assert lib.gq_linear_kn_workspace_bytes(1, 128, 64, 64) == 0  # one K slab: no scratch
-    assert lib.gq_linear_kn_workspace_bytes(300, 16384, 4096, 64) == 0  # prefill batches need none
-    assert lib.gq_linear_kn_workspace_bytes(48, 16384, 4096, 64) == 0
-    # ... unless they are expected to run faster as passes of the decode kernel over 16 rows each
-    assert lib.gq_linear_kn_workspace_bytes(17, 16384, 4096, 64) == lib.gq_linear_kn_workspace_bytes(16, 16384, 4096, 64) > 0
-    assert lib.gq_linear_kn_workspace_bytes(128, 4096, 16384, 64) == lib.gq_linear_kn_workspace_bytes(16, 4096, 16384, 64) > 0
+    assert lib.gq_linear_kn_workspace_bytes(300, 16384, 4096, 64) == 0  # prefill batches with tiles enough for the device need none
+    # ... with few tiles the prefill kernel divides K over workgroups: counters + 64 KiB per (slab, tile)
+    assert lib.gq_linear_kn_workspace_bytes(128, 16384, 4096, 64) == 16384 + 2 * 128 * 65536
+    assert lib.gq_linear_kn_workspace_bytes(300, 4096, 16384, 64) == 16384 + 3 * 96 * 65536
+    assert lib.gq_linear_kn_workspace_bytes(17, 16384, 4096, 64) == 16384 + 2 * 128 * 65536
     assert lib.gq_linear_kn_workspace_bytes(1, 16384, 4096, 20) == 0  # generic kernel
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 16384, 4096, 64, 0, None, 0, None)
