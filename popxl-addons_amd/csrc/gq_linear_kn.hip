@@ -417,6 +417,25 @@ bool kn_fast_shape(const uint16_t *x, const uint16_t *packed, int64_t n_out, int
 
 }  // namespace
 
+// K slabs of the prefill kernel: enough workgroups for the 256 compute units where the tiles alone are
+// few (a weight with 4096 outputs has 32 per 128 rows), slabs of at least 512 input features, at most 16
+int kn_prefill_splits(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t *slab_out) {
+  const int64_t tiles = ((n_out + BN - 1) / BN) * ((m_rows + BM - 1) / BM);
+  int64_t splits = tiles >= 192 ? 1 : (256 + tiles - 1) / tiles;
+  if (splits > 16) splits = 16;
+  if (splits > k_in / 512) splits = k_in / 512;
+  if (splits < 1 || tiles > kMaxStrips) splits = 1;
+  int64_t slab = (k_in + splits - 1) / splits;
+  slab = (slab + BK - 1) / BK * BK;
+  *slab_out = slab;
+  return (int)((k_in + slab - 1) / slab);
+}
+
+bool kn_prefill_shape(int64_t n_out, int64_t k_in, int64_t group_size) {
+  const bool pow2 = (group_size & (group_size - 1)) == 0;
+  return pow2 && group_size >= 32 && n_out % 32 == 0 && n_out >= 32 && n_out <= (int64_t)kMaxStrips * kStrip && k_in % BK == 0;
+}
+
 // Batches of 17 to 128 rows as passes of the decode kernel over 16 rows each, against the prefill
 // kernel, whose 128 x 128 tiles are mostly empty there.  From measured times (us): a pass of 16 rows
 // 18 + 0.37 per Mi weights (23.9 on 4096 -> 4096, 41.8 on 4096 -> 16384, 41.3 on 16384 -> 4096), fewer
