@@ -258,12 +258,17 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     x = torch.randn((m_rows, k_in), generator=g, device=device, dtype=torch.float32).to(torch.float16)
     y = torch.empty((m_rows, n_out), dtype=torch.float16, device=device)
     stream = stream_handle()
-    ws_bytes = hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, GROUP) if kn else 0
+    with_ws = entry == "gq_linear_act_ws_f16"  # (the layer's entry for the [n_out, k_in] layout: K may be divided over workgroups)
+    ws_bytes = (hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, GROUP) if kn else
+                hip.load().gq_gemm_workspace_bytes(m_rows, n_out, k_in, GROUP) if with_ws else 0)
     ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=device)
 
     def step(i):
         p, s, b = sets[i % n_sets]
         if kn:
+            hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP,
+                     0, ws.data_ptr(), ws.numel(), stream)
+        elif with_ws:
             hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP,
                      0, ws.data_ptr(), ws.numel(), stream)
         else:
@@ -650,9 +655,11 @@ def main():
         # batches between the GEMV's 16 rows and full GEMM tiles, through the entry that the layer calls
         extra["gemm_other_shapes"] = []
         for entry, m, n_out, k_in in (("gq_gemm_f16", 512, 4096, 4096), ("gq_gemm_f16", 512, 4096, 16384),
+                                      ("gq_linear_act_ws_f16", 128, 4096, 4096), ("gq_linear_act_ws_f16", 128, 4096, 16384),
+                                      ("gq_linear_act_ws_f16", 512, 4096, 16384),
                                       ("gq_linear_f16", 32, 4096, 4096), ("gq_linear_f16", 64, 16384, 4096)):
             r = bench_linear(hip, device, entry, m, n_out, k_in, 30, 5, n_sets=4,
-                             kernel="gemm_pipe2_kernel" if entry == "gq_gemm_f16" else "gemv_mfma_kernel passes / gemm_pipe2_kernel")
+                             kernel="gemm_pipe2_kernel" if entry != "gq_linear_f16" else "gemv_mfma_kernel passes / gemm_pipe2_kernel")
             r["entry"] = entry
             extra["gemm_other_shapes"].append(r)
             log(f"  {entry} m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s")

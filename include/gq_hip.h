@@ -127,6 +127,23 @@ int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed,
                       int64_t k_in, int64_t group_size, int32_t activation, void *stream);
 
 /*
+ * gq_linear_act_f16 with an optional workspace (no counterpart in the reference: LinearGQ.build has
+ * nothing to tune, popxl_addons/layers/linear_gq.py:99-109).  A weight with few outputs gives the
+ * GEMM kernel few output tiles (4096 outputs at 128 rows: 64 of 128 x 64 for 256 compute units);
+ * with the workspace, 2 to 16 workgroups divide the input features of a tile and add their binary32
+ * accumulators through it, in a fixed order.  gq_gemm_workspace_bytes() is the size for a problem
+ * (0: no division would pay, or m_rows <= 16); device memory, 16-byte aligned; its first 16 KiB hold
+ * arrival counters that the caller zeroes once and every call leaves zero, so one workspace serves
+ * calls of any shape -- one at a time: calls that share a workspace must not overlap.  A workspace
+ * that is NULL, misaligned or too small is not used: the call then is gq_linear_act_f16.
+ */
+int64_t gq_gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
+int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                         int64_t k_in, int64_t group_size, int32_t activation, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
+/*
  * Fused decompress + matmul, groups along the OUTPUT features: the computation of LinearGQ.build
  * with dim = -1 or 1, the constructor default (popxl_addons/layers/linear_gq.py:26, 59-62, 99-109):
  *   w = decompress(packed, scale, bias)      [k_in, n_out]

@@ -111,7 +111,7 @@ int gq_gemm_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   const int rc = gq::check_linear_args("gq_gemm_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
                                        k_in, group_size);
   if (rc <= 0) return rc;
-  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, GQ_ACT_NONE,
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, GQ_ACT_NONE, nullptr,
                          (hipStream_t)stream);
 }
 
@@ -127,19 +127,35 @@ int gq_linear_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, con
 int gq_linear_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                       const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                       int64_t group_size, int32_t activation, void *stream) {
+  return gq_linear_act_ws_f16(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, activation, nullptr, 0,
+                              stream);
+}
+
+int64_t gq_gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (m_rows <= 16) return 0;  // (the GEMV kernels take none)
+  return gq::gemm_workspace_bytes(m_rows, n_out, k_in, group_size);
+}
+
+int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
+                         int64_t group_size, int32_t activation, void *workspace, int64_t workspace_bytes, void *stream) {
   const int rc = gq::check_linear_args("gq_linear_act_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
                                        k_in, group_size);
   if (rc <= 0) return rc;
   if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_act_f16: unknown activation %d", (int)activation);
+  // the workspace is an option: one that is missing, misaligned or too small is not used
+  if (m_rows <= 16 || !workspace || gq::misaligned(workspace, 16) ||
+      workspace_bytes < gq_gemm_workspace_bytes(m_rows, n_out, k_in, group_size))
+    workspace = nullptr;
   if (m_rows <= 16)
     return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
                            (hipStream_t)stream);
   int passes_rc = GQ_OK;
   if (gq::launch_gemv_passes(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
-                             (hipStream_t)stream, &passes_rc))
+                             workspace != nullptr, (hipStream_t)stream, &passes_rc))
     return passes_rc;
-  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
+  return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation, workspace,
                          (hipStream_t)stream);
 }
 

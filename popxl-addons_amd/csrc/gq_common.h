@@ -37,15 +37,18 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream);
+// workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream);
+                int64_t group_size, int act, void *workspace, hipStream_t stream);
+int64_t gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
+double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split);
 // Batches of 17 to 128 rows as passes of the GEMV kernel over 16 rows each, where that is expected
 // to beat the GEMM kernel (whose 128 x 64 tiles are mostly empty there); false: not such a case,
 // nothing launched.
 bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                        int64_t group_size, int act, hipStream_t stream, int *rc);
+                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc);
 int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                              const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                              int64_t k_in, int64_t group_size, int act, hipStream_t stream);

@@ -267,7 +267,7 @@ template <int WM, int WN, int FM, int FN, int XS, int KS>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
-    int gs_shift, int act) {
+    int gs_shift, int act, float4_t *__restrict__ partial, unsigned *__restrict__ counters) {
   using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
   constexpr int NW = S::NW, TM = S::TM, TN = S::TN, TILE_M = S::TILE_M, TILE_N = S::TILE_N;
   constexpr int A_OPS = S::A_OPS, OPS = S::OPS;
@@ -279,8 +279,9 @@ __device__ __forceinline__ void gemm_pipe2_body(
   const int wm = wave / WN, wn = wave % WN;
   const int m0 = blockIdx.y * TILE_M, n0 = blockIdx.x * TILE_N;
   const int groups_per_row = k_in >> gs_shift;
-  const int n_tiles = (k_in >> 6) / KS;  // (the launcher checks divisibility)
-  const int tile0 = kgrp * n_tiles;
+  // gridDim.z > 1: the workgroups of an output tile divide K between them as well (see the end)
+  const int n_tiles = (k_in >> 6) / (KS * (int)gridDim.z);  // (the launcher checks divisibility)
+  const int tile0 = ((int)blockIdx.z * KS + kgrp) * n_tiles;
 
   const half_t *a_src[A_OPS];
 #pragma unroll
@@ -504,6 +505,60 @@ __device__ __forceinline__ void gemm_pipe2_body(
             acc[i][f][e] += red[((((g - 1) * NW + wave) * FM * FN + i * FN + f) * 16 + e) * 64 + lane];
   }
 
+  if (gridDim.z > 1) {
+    // K divided over the workgroups of the tile: their accumulators meet in `partial`
+    // ([slab][tile][wave][accumulator][quarter][lane], a float4 each); the last workgroup to arrive
+    // (arrival counters, zero before and after every launch) adds them in the order of the slabs.
+    // (The waves of the other K groups of this workgroup have left: barriers count the live waves.)
+    constexpr int kPerWave = FM * FN * 4;  // float4 per lane
+    const int n_splits = gridDim.z, tile = blockIdx.y * gridDim.x + blockIdx.x, n_out_tiles = gridDim.x * gridDim.y;
+    float4_t *mine = partial + (((int64_t)blockIdx.z * n_out_tiles + tile) * NW + wave) * (kPerWave * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int f = 0; f < FN; ++f)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const float4_t v = {acc[i][f][4 * q4], acc[i][f][4 * q4 + 1], acc[i][f][4 * q4 + 2], acc[i][f][4 * q4 + 3]};
+          asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(mine + ((i * FN + f) * 4 + q4) * 64), "v"(v) : "memory");
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial sums are in memory before the workgroup counts itself in
+    __builtin_amdgcn_s_barrier();
+    unsigned *arrived = reinterpret_cast<unsigned *>(lds);
+    if (tid == 0) {
+      const unsigned before = __hip_atomic_fetch_add(counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (before == (unsigned)n_splits - 1)  // the last one: leave the counter at zero for the next launch
+        __hip_atomic_store(counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(arrived, before, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __builtin_amdgcn_s_barrier();
+    if (__hip_atomic_load(arrived, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != (unsigned)n_splits - 1) return;
+    const float4_t *first = partial + ((int64_t)tile * NW + wave) * (kPerWave * 64) + lane;
+    const int64_t stride = (int64_t)n_out_tiles * NW * (kPerWave * 64);  // float4 between consecutive slabs
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int f = 0; f < FN; ++f)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][f][e] = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        float4_t v[FN * 4];
+#pragma unroll
+        for (int j = 0; j < FN * 4; ++j)
+          asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[j]) : "v"(first + sp * stride + (i * FN * 4 + j) * 64) : "memory");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < FN * 4; ++j) asm volatile("" : "+v"(v[j]));  // (uses of v stay below the wait)
+#pragma unroll
+        for (int f = 0; f < FN; ++f)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][f][e] += v[f * 4 + (e >> 2)][e & 3];
+      }
+    }
+  }
+
   // D[m][n]: lane holds n = lane % 32 and m = 8 * (e / 4) + 4 * (lane / 32) + e % 4
   const bool interior = m0 + TILE_M <= m_rows && n0 + TILE_N <= n_out;
 #pragma unroll
@@ -538,16 +593,20 @@ template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS>
 __global__ __launch_bounds__(KS * WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
                                                                   const half_t *scale, const half_t *bias,
                                                                   const half_t *out_bias, half_t *y, int n_out,
-                                                                  int k_in, int gs_shift, int act) {
-  gemm_pipe2_body<WM, WN, FM, FN, XS, KS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act);
+                                                                  int k_in, int gs_shift, int act, float4_t *partial,
+                                                                  unsigned *counters) {
+  gemm_pipe2_body<WM, WN, FM, FN, XS, KS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, partial,
+                                          counters);
 }
 
 namespace {
 
+constexpr int kGemmCounters = 4096;  // arrival counters at the start of a workspace (16 KiB), one per output tile
+
 template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS = 1>
 int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int gs_shift,
-                 int act, hipStream_t stream) {
+                 int act, int z_splits, void *workspace, hipStream_t stream) {
   using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
   constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
   static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
@@ -563,54 +622,115 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
     if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute(lds=%d): %s", lds_bytes, hipGetErrorString(e));
     configured[dev] = true;
   }
-  const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M));
+  const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M), (unsigned)z_splits);
   if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_gemm_f16: m_rows=%lld too large", (long long)m_rows);
+  unsigned *counters = static_cast<unsigned *>(workspace);
+  float4_t *partial = workspace ? reinterpret_cast<float4_t *>(counters + kGemmCounters) : nullptr;
   kern<<<grid, dim3(KS * WM * WN * 64), lds_bytes, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
-      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act);
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act, partial,
+      counters);
   return check_launch("gemm_pipe2_kernel");
 }
 
 }  // namespace
 
+namespace {
+
+// The tile shape and the number of workgroups that divide K for one output tile.
+//
+// Four tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
+// launch is as slow as its busiest compute unit: expected time = workgroups per compute unit (256 of
+// them; a last, partly filled round runs faster: fewer workgroups share memory and clocks) x time
+// per workgroup, from measured times per 1024 input features with every compute unit busy:
+//   64 x 64    6.3 us  (two groups of four waves of 32 x 32 that split K; needs k_in % 256 == 0)
+//   128 x 64   8 us    (16384 x 4096 at 128 rows: 34.5 us)
+//   256 x 128  22 us   (16384 x 4096 at 512 rows: 87 us; 16 us with an eighth of the compute units busy)
+//   256 x 256  34 us   (16384 x 4096 at 2048 rows: two rounds, 271 us; at 1024 rows one, 140 us)
+// Fixed thresholds on the batch alone (256 x 128 from 256 rows, 256 x 256 from 1024) left weights
+// with 4096 outputs on 16 to 64 workgroups: 4096 x 4096 at 512 rows took 75.6 us, now 36 us.  With each
+// shape forced in turn, this choice was the fastest or within 2 % of it for five weight shapes
+// (16384 x 4096, 4096 x 16384, 4096 x 4096, 12288 x 4096, 8192 x 8192) at nine batches from 128 to 4096.
+//
+// With a workspace, 2 to 16 workgroups may divide the K loop of a tile (each at least four steps of
+// 64) and add their fp32 accumulators through it: priced at 4 us plus the partial sums written and
+// read at 5 TB/s.
+struct GemmPlan {
+  int shape;   // 0: 64 x 64, 1: 128 x 64, 2: 256 x 128, 3: 256 x 256
+  int splits;  // workgroups per output tile
+  int64_t tiles, tile_bytes;
+  double us;   // expected time
+};
+
+GemmPlan plan_gemm(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split) {
+  static const int tile_m[4] = {64, 128, 256, 256}, tile_n[4] = {64, 64, 128, 256};
+  static const double us_per_1024[4] = {6.3, 8.0, 22.0, 34.0};
+  GemmPlan best = {1, 1, 0, 0, 1e30};
+  for (int shape = 3; shape >= 0; --shape) {  // (ties go to the larger tile)
+    if (shape == 0 && k_in % 256 != 0) continue;
+    const int groups = (shape <= 1 && k_in % 256 == 0) ? 2 : 1;  // groups of waves that split K inside a workgroup
+    const int64_t tiles = ((m_rows + tile_m[shape] - 1) / tile_m[shape]) * ((n_out + tile_n[shape] - 1) / tile_n[shape]);
+    for (int splits = 1; splits <= (may_split ? 16 : 1); splits *= 2) {
+      const int64_t steps = k_in / 64;
+      if (steps % (groups * splits) != 0 || steps / (groups * splits) < 4 || (splits > 1 && tiles > kGemmCounters)) break;
+      const int64_t wgs = tiles * splits, full = wgs / 256, rest = wgs % 256;
+      const int64_t tile_bytes = (int64_t)tile_m[shape] * tile_n[shape] * 4;
+      double t = ((double)full + (rest ? 0.7 + 0.3 * (double)rest / 256.0 : 0.0)) * us_per_1024[shape] * (double)k_in /
+                 (1024.0 * splits);
+      if (splits > 1) t += 4.0 + 2.0 * (double)(wgs * tile_bytes) / 5.0e6;
+      if (t < best.us) best = GemmPlan{shape, splits, tiles, tile_bytes, t};
+    }
+  }
+  return best;
+}
+
+bool gemm_pipelined_ok(const uint16_t *x, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, int64_t k_in,
+                       int64_t group_size) {
+  const bool pow2 = (group_size & (group_size - 1)) == 0;
+  if (!(pow2 && group_size >= 32 && k_in % BK == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)packed % 16) == 0))
+    return false;
+  // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
+  return (k_in / group_size) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0;
+}
+
+}  // namespace
+
+// What the choice above expects the pipelined kernel to take (us) -- for callers that weigh it against
+// other ways of running a batch.
+double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split) {
+  return plan_gemm(m_rows, n_out, k_in, may_split).us;
+}
+
+// Bytes of workspace with which launch_gemm may divide K over workgroups (0: it would not): 16 KiB of
+// arrival counters, then the fp32 accumulators of every (slab, tile).  (Pointer alignment is the
+// caller's to meet: this is the figure for 16-byte aligned operands.)
+int64_t gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
+  const bool pow2 = (group_size & (group_size - 1)) == 0;
+  if (m_rows < 1 || n_out < 1 || !pow2 || group_size < 32 || k_in <= 0 || k_in % BK != 0 || (k_in / group_size) % 2 != 0) return 0;
+  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, true);
+  return plan.splits == 1 ? 0 : (int64_t)kGemmCounters * 4 + plan.splits * plan.tiles * plan.tile_bytes;
+}
+
+// `workspace`: NULL, or gemm_workspace_bytes() bytes of device memory whose first 16 KiB (the counters)
+// are zero; the kernel leaves them zero.
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream) {
+                int64_t group_size, int act, void *workspace, hipStream_t stream) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % BK == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
   if (!fast_ok)
     return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
-#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...) \
-  launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, stream)
-  // the pipelined kernel fetches scale and bias as aligned dwords (two groups at a time)
-  if ((k_in >> gs_shift) % 2 == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0) {
-    // Four tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
-    // launch is as slow as its busiest compute unit: expected time = tiles per compute unit (256 of
-    // them; a last, partly filled round runs faster: fewer workgroups share memory and clocks) x
-    // time per tile, from measured times per 1024 input features with every compute unit busy:
-    //   128 x 64   8 us   (16384 x 4096 at 128 rows: 34.5 us)
-    //   256 x 128  22 us  (16384 x 4096 at 512 rows: 87 us; 16 us with an eighth of the compute units busy)
-    //   256 x 256  34 us  (16384 x 4096 at 2048 rows: two rounds, 271 us; at 1024 rows one, 140 us)
-    // Fixed thresholds on the batch alone (256 x 128 from 256 rows, 256 x 256 from 1024) left weights
-    // with 4096 outputs on 16 to 64 workgroups: 4096 x 4096 at 512 rows took 75.6 us, now 36 us.  With each
-    // shape forced in turn, this choice was the fastest or within 2 % of it for five weight shapes
-    // (16384 x 4096, 4096 x 16384, 4096 x 4096, 12288 x 4096, 8192 x 8192) at nine batches from 128 to 4096.
-    auto expected = [&](int tile_m, int tile_n, double us_per_1024) {
-      const int64_t tiles = ((m_rows + tile_m - 1) / tile_m) * ((n_out + tile_n - 1) / tile_n);
-      const int64_t full = tiles / 256, rest = tiles % 256;
-      return ((double)full + (rest ? 0.7 + 0.3 * (double)rest / 256.0 : 0.0)) * us_per_1024 * (double)k_in / 1024.0;
-    };
-    const double t_small = expected(128, 64, 8.0), t_mid = expected(256, 128, 22.0), t_large = expected(256, 256, 34.0);
-    // 64 x 64 (two groups of four waves of 32 x 32 that split K): 6.3 us per 1024 input features; for the
-    // batches and widths that leave the 128 x 64 tiles on half of the compute units or fewer (4096 x 4096
-    // at 256 rows: 26 against 31 us; 16384 x 4096 at 64 rows: 29 against 37 us)
-    const double t_tiny = k_in % 256 == 0 ? expected(64, 64, 6.3) : 1e30;
-    if (t_tiny < t_small && t_tiny < t_mid && t_tiny < t_large) return GQ_PIPE2(2, 2, 1, 1, 3, 2, 2);
-    if (t_large <= t_mid && t_large <= t_small) return GQ_PIPE2(1, 8, 8, 1, 4, 2);  // 256 x 256, 8 waves of 256 x 32
-    if (t_mid <= t_small) return GQ_PIPE2(1, 4, 8, 1, 3, 1);                        // 256 x 128, 4 waves of 256 x 32
+#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...)                                                                            \
+  launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, \
+                                                       plan.splits, plan.splits > 1 ? workspace : nullptr, stream)
+  if (gemm_pipelined_ok(x, packed, scale, bias, k_in, group_size)) {
+    const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, workspace != nullptr);
+    if (plan.shape == 0) return GQ_PIPE2(2, 2, 1, 1, 3, 2, 2);  // 64 x 64, two groups of 4 waves of 32 x 32
+    if (plan.shape == 3) return GQ_PIPE2(1, 8, 8, 1, 4, 2);     // 256 x 256, 8 waves of 256 x 32
+    if (plan.shape == 2) return GQ_PIPE2(1, 4, 8, 1, 3, 1);     // 256 x 128, 4 waves of 256 x 32
     // 128 x 64 (a workgroup on every compute unit at n_out = 16384), 4 waves of 64 x 32; two such
     // groups of waves split K when the K tiles divide between them (and the scale / bias dwords)
     if (k_in % 256 == 0) return GQ_PIPE2(2, 2, 2, 1, 3, 1, 2);

@@ -347,12 +347,12 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 // Passes of 16 rows against the GEMM kernel, from times measured on the three layer shapes of the 6B
 // stack (us): a pass takes 4.7 + 0.124 per Mi weights (6.8 on 4096 x 4096, 13.0 on 16384 x 4096; a
 // third more with rows of 8192 features or longer: 17.5 on 4096 x 16384); the GEMM kernel's 128 x 64
-// tiles take 7.5 per 1024 input features and round of 256 tiles (31 / 34 / 112 on the same shapes,
-// whatever the batch up to 128).  Measured: 4096 x 4096 at 32 rows 13.3 against 31.8, 4096 x 16384 at 64
+// tiles take 8 per 1024 input features and round of 256 tiles (31 / 34 / 112 on the same shapes,
+// whatever the batch up to 128; its own estimate is asked).  Measured: 4096 x 4096 at 32 rows 13.3 against 31.8, 4096 x 16384 at 64
 // rows 69.7 against 117.1, 16384 x 4096 at 32 rows 25.4 against 34.1 (and 38.0 against 35.2 at 48 rows).
 bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                        int64_t group_size, int act, hipStream_t stream, int *rc) {
+                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
@@ -360,10 +360,9 @@ bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packe
   const int64_t passes = (m_rows + 15) / 16;
   const double weights_mi = (double)n_out * (double)k_in / 1048576.0;
   const double t_pass = 4.7 + 0.124 * weights_mi * (k_in >= 8192 ? 1.35 : 1.0);
-  const int64_t tiles = (n_out + 63) / 64, tiles64 = tiles * ((m_rows + 63) / 64);
-  double t_gemm = 7.5 * ((double)k_in / 1024.0) * (double)((tiles + 255) / 256);
-  // (the GEMM kernel's 64 x 64 tiles, where it has them: 7 per 1024 input features and round of 256)
-  if (k_in % 256 == 0) t_gemm = std::min(t_gemm, 7.0 * ((double)k_in / 1024.0) * (double)((tiles64 + 255) / 256));
+  // (the GEMM kernel: what its own choice of tile -- and, with a workspace, of workgroups per tile -- expects)
+  const bool pipelined = (k_in / group_size) % 2 == 0 && k_in % 64 == 0;
+  const double t_gemm = pipelined ? gemm_expected_us(m_rows, n_out, k_in, gemm_may_split) : 1e30;
   if ((double)passes * t_pass >= t_gemm) return false;
   for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
     const int64_t m = m_rows - m0 < 16 ? m_rows - m0 : 16;

@@ -39,6 +39,8 @@ EXPORTS = (
     "gq_gemm_f16",
     "gq_linear_f16",
     "gq_linear_act_f16",
+    "gq_gemm_workspace_bytes",
+    "gq_linear_act_ws_f16",
     "gq_linear_kn_workspace_bytes",
     "gq_linear_kn_act_f16",
     "gq_linear_kn_act_noalloc_f16",
@@ -95,6 +97,10 @@ def load():
         fn.restype = ctypes.c_int
     lib.gq_linear_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p]
     lib.gq_linear_act_f16.restype = ctypes.c_int
+    lib.gq_gemm_workspace_bytes.argtypes = [i64, i64, i64, i64]
+    lib.gq_gemm_workspace_bytes.restype = i64
+    lib.gq_linear_act_ws_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
+    lib.gq_linear_act_ws_f16.restype = ctypes.c_int
     lib.gq_linear_kn_workspace_bytes.argtypes = [i64, i64, i64, i64]
     lib.gq_linear_kn_workspace_bytes.restype = i64
     lib.gq_linear_kn_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
@@ -137,7 +143,7 @@ _kn_workspaces = {}
 
 
 def linear_kn_workspace(device, nbytes):
-    """The scratch buffer of gq_linear_kn_act_f16 on `device` (one per device, grown on demand; its
+    """The scratch buffer of gq_linear_kn_act_f16 and gq_linear_act_ws_f16 on `device` (one per device, grown on demand; its
     arrival counters start at zero and every call leaves them zero).  Calls that share it are
     ordered by the stream they are enqueued on: use one stream per device for this layer."""
     import torch

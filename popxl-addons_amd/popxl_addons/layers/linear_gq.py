@@ -141,7 +141,11 @@ class LinearGQ:
             )
             stream = torch.cuda.current_stream(x.device).cuda_stream
             if self.dim == 0:
-                _gq_hip.call("gq_linear_act_f16", *args, stream)
+                # (few output tiles: several workgroups divide the input features of a tile through a workspace)
+                need = _gq_hip.load().gq_gemm_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)
+                ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None
+                _gq_hip.call("gq_linear_act_ws_f16", *args, 0 if ws is None else ws.data_ptr(),
+                             0 if ws is None else ws.numel(), stream)
             else:
                 # groups along the output features: weight rows are input features
                 need = _gq_hip.load().gq_linear_kn_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)

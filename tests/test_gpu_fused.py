@@ -196,6 +196,38 @@ def test_gemm_large_tiles_on_ragged_problems(hip, device, oracle, n_out, k_in, m
     assert_close(y, y_ref, (n_out, k_in, m_rows))
 
 
+def test_linear_with_workspace(hip, device, oracle):
+    """gq_linear_act_ws_f16: on weights with few outputs the workgroups of an output tile divide the
+    input features between them and add their accumulators through the workspace.  One workspace
+    serves problems of several shapes one after the other (its arrival counters are back at zero after
+    every call); ragged tiles, every tile shape that the choice reaches here, an activation; the
+    result is the oracle's, and that of the call without a workspace to a few roundings."""
+    lib = hip.load()
+    cases = [(4096, 16384, 128), (4096, 16384, 300), (4096, 4096, 64), (4096, 4096, 256), (4104, 2048, 100), (2056, 8192, 520),
+             (1000, 4096, 40)]
+    needs = [lib.gq_gemm_workspace_bytes(m, n, k, 64) for n, k, m in cases]
+    assert sum(need > 16384 for need in needs) >= 5, needs  # (a problem for which dividing K does not pay asks for none)
+    assert lib.gq_gemm_workspace_bytes(16, 4096, 16384, 64) == 0 and lib.gq_gemm_workspace_bytes(2048, 16384, 4096, 64) == 0
+    ws = torch.zeros(max(needs), dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream().cuda_stream
+    for (n_out, k_in, m_rows), need in zip(cases, needs):
+        x, packed, scale, bias, ob, _ = _case(oracle, n_out, k_in, 64, m_rows, 29, True)
+        w_dec = _CASE_WEIGHTS[(n_out, k_in, 64, 29)][3]
+        y_ref = oracle.np_linear(x, w_dec, ob, "gelu_tanh")
+        xd, pd, sd, bd, od = (to_dev(a, device) for a in (x, packed, scale, bias, ob))
+        got = []
+        for workspace in (ws, None):
+            y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+            hip.call("gq_linear_act_ws_f16", xd.data_ptr(), m_rows, pd.data_ptr(), sd.data_ptr(), bd.data_ptr(), od.data_ptr(),
+                     y.data_ptr(), n_out, k_in, 64, 2, 0 if workspace is None else workspace.data_ptr(),
+                     0 if workspace is None else workspace.numel(), stream)
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), y_ref, (n_out, k_in, m_rows, workspace is not None))
+            got.append(y.cpu().numpy())
+        assert not ws[:16384].any(), "arrival counters must be back at zero"
+        assert normalised_error(got[0], got[1].astype(np.float32)) <= REGRESSION_TOL
+
+
 @pytest.mark.parametrize("m_rows", [33, 70, 100, 260, 300, 1030])
 def test_gemm_every_kernel_shape(hip, device, oracle, m_rows):
     """Small ragged problems on the pipelined kernel's 128 x 64 tiles (with K split between two groups
