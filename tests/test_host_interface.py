@@ -30,6 +30,15 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, n) is not None
 
 
+def test_every_entry_point_has_its_reference_interface_written_down():
+    """The integration notes name, for every declared entry point, the reference interface it stands
+    for (or say that it has none), and name no entry point that does not exist."""
+    with open(os.path.join(ROOT, "INTEGRATION.md")) as f:
+        table = [line for line in f if line.startswith("| `gq_")]
+    listed = set(re.findall(r"`(gq_[a-z0-9_]+)`", " ".join(line.split("|")[1] for line in table)))
+    assert listed == set(_declared_functions())
+
+
 def test_abi_version_and_error_text_without_gpu():
     lib = _gq_hip.load()
     assert lib.gq_abi_version() == _gq_hip.GQ_ABI_VERSION
