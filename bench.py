@@ -8,9 +8,10 @@ configuration 2: group 64, ~N(0, 0.02) with 0.1 % outliers at +-8 sigma, packed 
 device-side packer that the tests hold bit-identical to the numpy packer).  Inputs are resident in
 HBM before the timed region; buffer sets are rotated so that the working set (4 x 172 MB) does not
 fit the 256 MB last-level cache.  The fused GEMV / GEMM / layer-stack measurements of the other
-configurations are reported in the same JSON line under "extra".
+configurations are summarised in the same JSON line under "extra" (one short record per shape);
+every figure of the run goes to the detail file (default gpurun_out/bench_detail.json) and to stderr.
 
-Prints ONE JSON line on stdout; progress goes to stderr.
+The LAST line on stdout is the one JSON line (under 4 KB); progress goes to stderr.
 """
 import argparse
 import json
@@ -242,6 +243,12 @@ def cpu_baseline_legs():
 # -------------------------------------------------------------------------------------- fused
 
 
+def sets_beyond_cache(n_out, k_in):
+    """Distinct weights to rotate over so that their packed bytes (> 600 MB) cannot stay in the
+    256 MB last-level cache from one launch to the next."""
+    return max(2, int(600e6 // (n_out * k_in * (0.5 + 4.0 / GROUP))) + 1)
+
+
 def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets, kernel):
     """One fused dequant matmul shape; weights rotated over n_sets distinct copies.  `entry` is
     gq_gemv_f16 / gq_gemm_f16 (weight [n_out, k_in], groups along k_in) or gq_linear_kn_act_f16
@@ -279,7 +286,7 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     w_bytes = n_out * k_in * (0.5 + 4.0 / GROUP)
     flops = 2.0 * m_rows * n_out * k_in
     r = {
-        "m": m_rows, "n": n_out, "k": k_in, "layout": "[k_in, n_out]" if kn else "[n_out, k_in]", "us": ms * 1e3,
+        "m": m_rows, "n": n_out, "k": k_in, "layout": "[k_in, n_out]" if kn else "[n_out, k_in]", "n_sets": n_sets, "us": ms * 1e3,
         "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
         "tflops": flops / ms / 1e9, "mfma_frac": flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS,
     }
@@ -537,6 +544,85 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
     return results
 
 
+# ------------------------------------------------------------------------------------ output
+HEADLINE_LIMIT = 4096  # bytes: the final stdout line must stay a line that a log capture keeps whole
+
+# the decoder schedules of the stack, best first where several ran: what "decoder" means in the headline
+DECODER_MODES = ("sequence_decoder_data_flow_two_entries_streaming_layout", "sequence_decoder_data_flow_joint_output_streaming_layout",
+                 "sequence_decoder_data_flow_streaming_layout", "sequence_decoder_data_flow",
+                 "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", "sequence_parallel_block_fused_qkv_ffn_first")
+
+
+def _row(r, frac_key):
+    return {"m": r["m"], "n": r["n"], "k": r["k"], "us": round(r["us"], 1), "frac": round(r[frac_key], 3)}
+
+
+def _stack_summary(r):
+    """One record per batch of the 28-layer stack: the fastest decoder schedule that ran, the same
+    kernel without dependencies, and one launch per matrix replayed from a graph."""
+    out = {"m": r["m"]}
+    ran = [(r[mode]["us_per_pass"], mode) for mode in DECODER_MODES if mode in r]
+    if ran:
+        us, mode = min(ran)
+        out["decoder"] = {"us": round(us), "frac": round(r[mode]["hbm_frac"], 3), "kernel": r[mode]["roofline"]["kernel"],
+                          "schedule": mode.replace("sequence_", "")}
+    for key, mode in (("no_waits", "sequence_no_waits_streaming_layout"), ("per_launch_graph", "per_launch_graph"),
+                      ("default_layout", "default_layout_graph"), ("default_layout_sequence", "default_layout_sequence")):
+        if mode in r:
+            out[key] = {"us": round(r[mode]["us_per_pass"]), "frac": round(r[mode]["hbm_frac"], 3)}
+    return out
+
+
+def headline(result):
+    """The line for stdout: the top-level keys as they are, `roofline`, `cpu_baseline` without its
+    legs, and under `extra` one short record per benchmark shape (microseconds, fraction of the
+    roofline that bounds it).  Everything else stays in the detail file."""
+    extra = result.get("extra") or {}
+    short = {k: extra[k] for k in ("detail_file", "gpu_equals_cpu_baseline_bits", "bench_wall_s") if k in extra}
+    if any(k in extra for k in ("gemv", "linear_kn", "gemm")):
+        short["weights"] = "every row rotates over distinct weights of > 600 MB packed bytes in total (n_sets in the detail file)"
+    for key in ("decompress_transposed", "compress", "compress_f32"):
+        if key in extra:
+            short[key] = {"us": round(extra[key]["us"], 1), "frac": round(extra[key]["hbm_frac"], 3)}
+    if "gemv" in extra:  # configuration 3 (+ the stack's third shape): fraction of HBM peak on the packed weight
+        short["c3_gemv"] = [_row(r, "hbm_frac") for r in extra["gemv"]]
+    if "linear_kn" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out])
+        short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] <= 16]
+        short["gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
+    if "gemm" in extra:  # configuration 4: fraction of the dense fp16 MFMA peak
+        short["c4_gemm"] = [_row(r, "mfma_frac") for r in extra["gemm"]]
+    if "stack" in extra:  # configuration 5: fraction of HBM peak on the packed weight
+        short["c5_stack"] = [_stack_summary(r) for r in extra["stack"]]
+    out = {k: v for k, v in result.items() if k not in ("extra", "cpu_baseline", "roofline")}
+    roof = dict(result["roofline"])
+    roof.pop("traffic_source", None)
+    out["roofline"] = roof
+    cpu = result.get("cpu_baseline")
+    out["cpu_baseline"] = None if cpu is None else {k: v for k, v in cpu.items() if k != "legs"}
+    out["extra"] = short
+    return out
+
+
+def emit(result, detail_path):
+    """Detail to its file and to stderr, the headline as the last line of stdout."""
+    if detail_path:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(detail_path)), exist_ok=True)
+            with open(detail_path, "w") as f:
+                json.dump(result, f, indent=1)
+            result["extra"]["detail_file"] = os.path.relpath(detail_path, ROOT) if os.path.abspath(detail_path).startswith(ROOT) else detail_path
+        except OSError as e:  # (a read-only tree: the detail still goes to stderr)
+            log(f"bench.py: could not write {detail_path}: {e}")
+    log("detail: " + json.dumps(result))
+    line = json.dumps(headline(result), separators=(",", ":"))
+    if len(line) >= HEADLINE_LIMIT:  # never expected (a test holds the size on a full run's detail): drop the per-shape records
+        slim = headline(result)
+        slim["extra"] = {k: v for k, v in slim["extra"].items() if not isinstance(v, list)}
+        line = json.dumps(slim, separators=(",", ":"))
+    sys.stderr.flush()
+    print(line, flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -547,6 +633,8 @@ def main():
     ap.add_argument("--stack-modes", default="",
                     help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
     ap.add_argument("--stack-batches", default="1,4", help="batch sizes of the stack runs")
+    ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+                    help="file for every figure of the run (the stdout line holds a summary); empty: no file")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB device copy (known traffic) for scaling profiler byte counters")
     args = ap.parse_args()
@@ -626,7 +714,7 @@ def main():
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
             for m in (1, 8):
                 r = bench_linear(hip, device, "gq_gemv_f16", m, n_out, k_in, 200, 20,
-                                 n_sets=max(2, int(600e6 // (n_out * k_in * 0.5625)) + 1), kernel="gemv_mfma_kernel / gemv_stream_single_kernel")
+                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_mfma_kernel / gemv_stream_single_kernel")
                 extra["gemv"].append(r)
                 log(f"  gemv m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
@@ -636,18 +724,19 @@ def main():
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
             for m in (1, 8):
                 r = bench_linear(hip, device, "gq_linear_kn_act_f16", m, n_out, k_in, 200, 20,
-                                 n_sets=max(2, int(600e6 // (n_out * k_in * 0.5625)) + 1), kernel="gemv_kn_kernel")
+                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_kn_kernel")
                 extra["linear_kn"].append(r)
                 log(f"  kn-layout gemv m={m} [{k_in}->{n_out}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
-        r = bench_linear(hip, device, "gq_linear_kn_act_f16", 128, 16384, 4096, 30, 5, n_sets=2, kernel="gemm_kn_tile_kernel")
+        r = bench_linear(hip, device, "gq_linear_kn_act_f16", 128, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096), kernel="gemm_kn_tile_kernel")
         extra["linear_kn"].append(r)
         log(f"  kn-layout gemm m=128 [4096->16384]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
         torch.cuda.empty_cache()
     if args.only in ("gemm", "all"):
         extra["gemm"] = []
         for m in (128, 512, 2048):
-            r = bench_linear(hip, device, "gq_gemm_f16", m, 16384, 4096, 30, 5, n_sets=2, kernel="gemm_pipe2_kernel")
+            # (weights out of HBM at every batch: 17 distinct 16384 x 4096 weights, 641 MB of packed bytes)
+            r = bench_linear(hip, device, "gq_gemm_f16", m, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096), kernel="gemm_pipe2_kernel")
             extra["gemm"].append(r)
             log(f"  gemm m={m} [16384x4096]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
             torch.cuda.empty_cache()
@@ -658,7 +747,7 @@ def main():
                                       ("gq_linear_act_ws_f16", 128, 4096, 4096), ("gq_linear_act_ws_f16", 128, 4096, 16384),
                                       ("gq_linear_act_ws_f16", 512, 4096, 16384),
                                       ("gq_linear_f16", 32, 4096, 4096), ("gq_linear_f16", 64, 16384, 4096)):
-            r = bench_linear(hip, device, entry, m, n_out, k_in, 30, 5, n_sets=4,
+            r = bench_linear(hip, device, entry, m, n_out, k_in, 60, 5, n_sets=sets_beyond_cache(n_out, k_in),
                              kernel="gemm_pipe2_kernel" if entry != "gq_linear_f16" else "gemv_mfma_kernel passes / gemm_pipe2_kernel")
             r["entry"] = entry
             extra["gemm_other_shapes"].append(r)
@@ -712,7 +801,7 @@ def main():
         "cpu_baseline": cpu,
         "extra": extra,
     }
-    print(json.dumps(result), flush=True)
+    emit(result, args.detail)
 
 
 if __name__ == "__main__":
