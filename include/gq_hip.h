@@ -17,9 +17,16 @@
  *     (nothing was launched); a positive value is a `hipError_t` from the runtime.
  *     `gq_last_error()` returns a thread-local, human-readable description of the last
  *     non-zero return on the calling thread.
- *   - Functions are re-entrant, allocate nothing and keep no state between calls (one exception:
- *     gq_gemv_sequence_f16 uses a block of progress words that the library keeps per device, see
- *     there); there are no process-wide options.  Every entry point can be captured in a HIP graph.
+ *   - Functions allocate nothing and there are no process-wide options.  What the library keeps
+ *     between calls, per device: (1) the block of progress words and exchange buffers of
+ *     gq_gemv_sequence_f16, (2) the scratch array of gq_linear_kn_act_noalloc_f16, (3) for kernels
+ *     that need more than 64 KiB of LDS, the fact that hipFuncSetAttribute has been called for them
+ *     (set on first use, never changed).  (1) and (2) are shared by every call on the device: such
+ *     calls must be enqueued on ONE stream per device; a call that arrives on another stream while
+ *     the previous one's stream still has work pending returns GQ_ERR_UNSUPPORTED and launches
+ *     nothing (streams under capture are not checked: ordering graph replays is the caller's job).
+ *     Their siblings that take a workspace (gq_gemv_sequence_ws_f16, gq_linear_kn_act_f16) keep
+ *     nothing.  All other functions are re-entrant.  Every entry point can be captured in a HIP graph.
  *
  * Packed layout (group_quantize_decompress.py:127-135, group_quantize_decompress_codelet.cpp:11-14)
  *   packed[r][g][i] is a little-endian uint16 holding four 4-bit codes, most significant
@@ -191,6 +198,9 @@ int gq_linear_kn_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
  * fit, the prefill kernel, which needs no scratch, runs (the same result to the tolerance of the
  * fused paths, not bit for bit).
  * All calls on one GPU share the array: calls that overlap on one GPU (different streams) race.
+ * Enqueue them on one stream per GPU: a call on another stream while the previous call's stream
+ * still has work pending returns GQ_ERR_UNSUPPORTED (nothing launched); calls under stream capture
+ * are not checked.
  */
 #define GQ_LINEAR_KN_NOALLOC_PARTIAL_BYTES (4 << 20)
 int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
@@ -231,6 +241,9 @@ int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16
  *
  * gq_gemv_sequence_f16     keeps the per-workgroup progress words in a block that the library
  *                          holds per device: at most ONE sequence may run on a device at a time.
+ *                          Calls are ordered by their stream; a call on a different stream while the
+ *                          stream of the previous call still has work pending is refused with
+ *                          GQ_ERR_UNSUPPORTED (nothing launched) rather than left to corrupt both.
  * gq_gemv_sequence_ws_f16  takes them from `workspace` (device memory, 256-byte aligned,
  *                          gq_gemv_sequence_workspace_bytes() bytes -- progress words and the
  *                          buffers through which results travel from entry to entry inside a

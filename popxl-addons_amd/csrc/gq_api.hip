@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "gq_common.h"
 
@@ -25,6 +26,28 @@ int check_launch(const char *what) {
   const hipError_t e = hipGetLastError();
   if (e == hipSuccess) return GQ_OK;
   return fail((int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+int claim_shared_block(SharedBlockGuard &guard, int dev, hipStream_t stream, const char *who) {
+  static std::mutex lock;
+  if (dev < 0 || dev >= SharedBlockGuard::kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "%s: device index %d", who, dev);
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) (void)hipGetLastError();
+  if (capture != hipStreamCaptureStatusNone) return GQ_OK;
+  std::lock_guard<std::mutex> hold(lock);
+  if (guard.used[dev] && guard.last[dev] != stream) {
+    // (a stream that no longer exists gives an error code: nothing of it can be pending)
+    const hipError_t pending = hipStreamQuery(guard.last[dev]);
+    (void)hipGetLastError();  // the query's "not ready" is an answer, not an error of this call
+    if (pending == hipErrorNotReady)
+      return fail(GQ_ERR_UNSUPPORTED,
+                  "%s: the block that the library keeps per device is still in use by work enqueued on another stream; "
+                  "calls that share it must be enqueued on one stream (or the other stream's work must have completed) -- "
+                  "use the variant that takes a workspace for concurrent streams", who);
+  }
+  guard.last[dev] = stream;
+  guard.used[dev] = true;
+  return GQ_OK;
 }
 
 namespace {

@@ -12,6 +12,19 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // Maps the runtime's last launch error (if any) to a return code, recording its text.
 int check_launch(const char *what);
 
+// A block of device memory that the library keeps per GPU and every call on that GPU shares (the
+// progress words of gq_gemv_sequence_f16, the scratch of gq_linear_kn_act_noalloc_f16): calls
+// that use it are ordered by the stream they are enqueued on.  Remembers the stream of the last
+// call per device; a call on ANOTHER stream while that stream still has work pending is refused
+// (GQ_ERR_UNSUPPORTED, nothing launched) instead of racing silently.  A stream under capture is
+// neither checked nor remembered (replays of a graph are the caller's to order).
+struct SharedBlockGuard {
+  static constexpr int kMaxDevices = 64;
+  hipStream_t last[kMaxDevices];
+  bool used[kMaxDevices];
+};
+int claim_shared_block(SharedBlockGuard &guard, int dev, hipStream_t stream, const char *who);
+
 typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));

@@ -1017,12 +1017,7 @@ void plan_launch(const gq_gemv_desc *e, int n, int64_t first, bool any_fit, int 
 }  // namespace
 
 // launches of weights in the streaming layout whose dependencies all travel through the exchange
-// run on the data-flow kernel of gq_gemv_flow.hip (a build without it, for comparisons: -DGQ_NO_FLOW)
-#ifdef GQ_NO_FLOW
-constexpr bool kUseFlow = false;
-#else
-constexpr bool kUseFlow = true;
-#endif
+// run on the data-flow kernel of gq_gemv_flow.hip
 
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
                          void *workspace, int64_t spin_limit, hipStream_t stream) {
@@ -1054,6 +1049,9 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
   unsigned *words = static_cast<unsigned *>(workspace);
   if (!words) {
     // the library's own block of this device (its address differs from device to device)
+    static SharedBlockGuard guard = {};
+    const int claimed = claim_shared_block(guard, dev, stream, "gq_gemv_sequence_f16");
+    if (claimed != GQ_OK) return claimed;
     static unsigned *own[kMaxDevices] = {nullptr};
     if (!own[dev]) {
       void *ptr = nullptr;
@@ -1079,13 +1077,11 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
       const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
       SequencePlan plan;                                                                                      \
-      if (kUseFlow) {                                                                                         \
-        plan_launch(host + first, n, first, true, grid, plan);                                                      \
-        if (flow_eligible(host + first, n, plan)) {                                                           \
-          const int rc = launch_flow(host + first, device + first, n, status, words, spins, plan, grid, dev, stream); \
-          if (rc != GQ_OK) return rc;                                                                         \
-          continue;                                                                                           \
-        }                                                                                                     \
+      plan_launch(host + first, n, first, true, grid, plan);                                                  \
+      if (flow_eligible(host + first, n, plan)) {                                                             \
+        const int rc = launch_flow(host + first, device + first, n, status, words, spins, plan, grid, dev, stream); \
+        if (rc != GQ_OK) return rc;                                                                           \
+        continue;                                                                                             \
       }                                                                                                       \
       plan_launch(host + first, n, first, false, grid, plan);                                                 \
       kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status, words, spins, plan); \

@@ -573,6 +573,9 @@ int launch_linear_kn_noalloc(const uint16_t *x, int64_t m_rows, const uint16_t *
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fail((int)e, "hipGetDevice: %s", hipGetErrorString(e));
     if (dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_UNSUPPORTED, "device index %d", dev);
+    static SharedBlockGuard guard = {};
+    const int claimed = claim_shared_block(guard, dev, stream, "gq_linear_kn_act_noalloc_f16");
+    if (claimed != GQ_OK) return claimed;
     if (!scratch_ptr[dev]) {
       void *p = nullptr;
       e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));

@@ -143,15 +143,23 @@ _kn_workspaces = {}
 
 
 def linear_kn_workspace(device, nbytes):
-    """The scratch buffer of gq_linear_kn_act_f16 and gq_linear_act_ws_f16 on `device` (one per device, grown on demand; its
-    arrival counters start at zero and every call leaves them zero).  Calls that share it are
-    ordered by the stream they are enqueued on: use one stream per device for this layer."""
+    """The scratch buffer of gq_linear_kn_act_f16 and gq_linear_act_ws_f16 for calls enqueued on the
+    CURRENT stream of `device`: one buffer per (device, stream), grown on demand; its arrival counters
+    start at zero and every call leaves them zero.  Calls that share a buffer are on the same stream
+    and therefore ordered; layers built on different streams get different buffers and may overlap."""
     import torch
 
-    ws = _kn_workspaces.get(device)
+    device = torch.device(device)
+    if device.index is None:
+        device = torch.device(device.type, torch.cuda.current_device())
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _kn_workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-        _kn_workspaces[device] = ws
+        with torch.cuda.device(device):
+            # (a buffer that is being replaced stays alive until the work enqueued on it has run:
+            # the caching allocator hands its memory out again on the same stream only)
+            ws = torch.zeros(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _kn_workspaces[key] = ws
     return ws
 
 
@@ -189,14 +197,23 @@ class GemvSequence:
     entry from torch tensors on the GPU (kept alive by this object) and returns its index; the entry
     starts after every earlier entry (wait_previous) or after entries 0..wait_for have completed.
     run() enqueues the whole list on the current stream.  `status` is a device int32 the kernel
-    sets to 1 if it gave up waiting.
+    sets to 1 if it gave up waiting (some workgroup of the persistent kernel was not resident:
+    another kernel held compute units); the results of that run are then invalid.  A give-up does
+    not pass silently: run() raises GQHipError as soon as it finds that an earlier run() of this
+    object ended that way (it looks at a host copy of `status` that earlier runs left behind, without
+    waiting for the GPU), and check() waits for the GPU and raises for every run so far.  After the
+    error has been raised once the object is usable again.
     """
 
     def __init__(self, device, own_workspace=False, spin_limit=0):
         """own_workspace: keep the kernel's progress words in a buffer of this object
-        (gq_gemv_sequence_ws_f16) instead of the block the library holds per device, so that
-        several sequences may be enqueued on different streams; spin_limit: polls without
-        progress after which a wait gives up (0: the library's default)."""
+        (gq_gemv_sequence_ws_f16) instead of the block the library holds per device.  Sequences
+        with buffers of their own may be enqueued on different streams, but the caller must still
+        ORDER them (events): each persistent kernel needs every compute unit, and two that really
+        overlap give up (status 1).  Without it, all sequences of a device share the library's block
+        and must be enqueued on one stream (the library refuses a second stream while the first is
+        busy).  spin_limit: polls without progress after which a wait gives up (0: the library's
+        default)."""
         import numpy as np
 
         self.device = device
@@ -214,6 +231,8 @@ class GemvSequence:
         self._host = None
         self._dev = None
         self.status = None
+        self._status_host = None   # pinned int32: the last copy of `status` that reached the host
+        self._status_event = None  # recorded behind that copy; None: no copy under way
 
     def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None, activation=None):
         """`packed` may be a PrepackedWeight (then scale and bias are None)."""
@@ -252,6 +271,8 @@ class GemvSequence:
         self._host = np.array(self.entries, dtype=self.dtype)
         self._dev = torch.from_numpy(self._host.view(np.uint8).copy()).to(self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._status_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self._status_event = None
         if self.own_workspace and self._workspace is None:
             self._workspace = torch.zeros(load().gq_gemv_sequence_workspace_bytes(), dtype=torch.uint8, device=self.device)
 
@@ -260,6 +281,9 @@ class GemvSequence:
 
         if self._host is None:
             self._finalise()
+        capturing = torch.cuda.is_current_stream_capturing()
+        if not capturing:
+            self._raise_if_gave_up(wait=False)
         stream = torch.cuda.current_stream(self.device).cuda_stream
         if self.own_workspace:
             call("gq_gemv_sequence_ws_f16", self._host.ctypes.data, self._dev.data_ptr(), len(self.entries),
@@ -267,13 +291,37 @@ class GemvSequence:
         else:
             call("gq_gemv_sequence_f16", self._host.ctypes.data, self._dev.data_ptr(), len(self.entries),
                  self.status.data_ptr(), stream)
+        # `status` only ever goes from 0 to 1 on the device, so any later copy also tells of this run.  One
+        # copy at a time: a loop that enqueues runs faster than the GPU executes them adds no copies.
+        if not capturing and self._status_event is None:
+            self._status_host.copy_(self.status, non_blocking=True)
+            self._status_event = torch.cuda.Event()
+            self._status_event.record(torch.cuda.current_stream(self.device))
 
-    def check(self):
-        """Synchronise and raise if a wait of the last run() gave up (results are then invalid)."""
+    _GAVE_UP = ("a wait for earlier entries gave up, the results of that run are invalid: some workgroup was not "
+                "resident (is another kernel occupying the compute units?)")
+
+    def _raise_if_gave_up(self, wait):
         import torch
 
-        torch.cuda.synchronize(self.device)
-        if self.status is not None and int(self.status.item()) != 0:
+        if self.status is None:
+            return
+        if wait:
+            torch.cuda.synchronize(self.device)
+            gave_up = int(self.status.item()) != 0
+            self._status_event = None
+        else:
+            if self._status_event is None or not self._status_event.query():
+                return
+            self._status_event = None
+            gave_up = int(self._status_host[0]) != 0
+        if gave_up:
+            torch.cuda.synchronize(self.device)
             self.status.zero_()
-            raise GQHipError("gq_gemv_sequence_f16", 1, "a wait for earlier entries gave up: some workgroup was not "
-                             "resident (is another kernel occupying the compute units?)")
+            self._status_host.zero_()
+            torch.cuda.synchronize(self.device)
+            raise GQHipError("gq_gemv_sequence_f16", 1, self._GAVE_UP)
+
+    def check(self):
+        """Wait for the GPU and raise if a wait of any run() so far gave up (results are then invalid)."""
+        self._raise_if_gave_up(wait=True)

@@ -251,11 +251,12 @@ class LinearGQ:
 
         dtype = torch.float32 if dtype is None else dtype
         weight_t = nn_layer.weight.T.detach()
-        if weight_t.is_cuda:
+        if weight_t.is_cuda and weight_t.dtype in (torch.float16, torch.float32):
             # the packer on the device: the same bits as the numpy function gives for this array
             compressed = tuple(a.cpu().numpy() for a in group_quantize_compress(weight_t, group_size, dim=dim))
         else:
-            compressed = group_quantize_compress_numpy(weight_t.numpy(), group_size, dim=dim)
+            # (any other dtype, e.g. float64: the numpy packer, as the reference does for every weight)
+            compressed = group_quantize_compress_numpy(weight_t.cpu().numpy(), group_size, dim=dim)
         state_dict = dict(
             zip(
                 (

@@ -885,3 +885,161 @@ def test_gemv_sequence_decoder_schedule_at_full_size(hip, device, oracle, m_rows
         shared_seq.check()
         for want, (_, _, y) in zip(final, shared_plan[-4:]):
             assert torch.equal(want, y), run
+
+
+# --------------------------------------------------------------------------------------------------
+# the benchmark's own 28-layer schedules, and what happens when a sequence cannot finish
+
+
+def test_benchmark_stack_28_layers_against_oracle(hip, device, oracle):
+    """The exact 28-layer schedules that bench.py times at one batch row (four entries per layer and
+    two entries per layer, every weight in the streaming layout, 3.17 GB of packed weights): after the
+    passes, the last layer's outputs equal the oracle's linear over the oracle-decompressed weights,
+    applied to the inputs the device had -- 27 layers of ring wrap-around, result exchange and
+    launches of 112 / 56 entries lie in front of them.  bench.py does the comparison when it is
+    handed the oracle (it raises if the error exceeds 1e-2 or the kernel gave up)."""
+    import bench
+
+    modes = ("sequence_decoder_data_flow_streaming_layout", "sequence_decoder_data_flow_two_entries_streaming_layout",
+             "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout")
+    r = bench.bench_stack(hip, device, 1, passes=3, warmup=1, modes=modes, oracle=oracle)
+    for mode in modes:
+        assert r[mode]["status"] == 0
+        assert r[mode]["max_error_vs_oracle"] <= REGRESSION_TOL, (mode, r[mode])
+        assert r[mode]["max_error_vs_single_call"] <= REGRESSION_TOL, (mode, r[mode])
+    torch.cuda.empty_cache()
+
+
+def test_benchmark_stack_28_layers_batch_4_against_oracle(hip, device, oracle):
+    """The same at four batch rows (the LDS-ring kernel)."""
+    import bench
+
+    modes = ("sequence_decoder_data_flow_streaming_layout",)
+    r = bench.bench_stack(hip, device, 4, passes=2, warmup=1, modes=modes, oracle=oracle)
+    assert r[modes[0]]["status"] == 0 and r[modes[0]]["max_error_vs_oracle"] <= REGRESSION_TOL, r[modes[0]]
+    torch.cuda.empty_cache()
+
+
+def _chained_streaming_case(hip, device, oracle, shapes, seed):
+    """Chained entries at one batch row, every weight in the streaming layout: (entries, oracle results)."""
+    from popxl_addons._gq_hip import prepack_gemv
+
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, 1, chained=True, seed=seed)
+    entries = [(x, prepack_gemv(packed, scale, bias), y, ob) for x, packed, scale, bias, y, ob in seq.keep]
+    return entries, seq, refs, outs
+
+
+def _assert_chain(oracle, seq, refs, outs):
+    x_prev = None
+    for i, y in enumerate(outs):
+        yy = y.cpu().numpy()
+        if i == 0:
+            assert_close(yy, refs[0])
+        else:
+            e = seq.keep[i]
+            w_dec = oracle.np_decompress(e[1].cpu().numpy(), e[2].cpu().numpy(), e[3].cpu().numpy())
+            assert_close(yy, oracle.np_linear(x_prev, w_dec, None if e[5] is None else e[5].cpu().numpy()), i)
+        x_prev = yy
+
+
+# word index of the data-flow kernel's launch count in a sequence workspace: 256 progress lines, the
+# announcement, the exit count and the epoch (a 128-byte line each), rounded up to 256 bytes, then the
+# 16 MiB exchange of the other kernel
+_FLOW_EPOCH_WORD = ((256 + 3) * 32 + 32 + 63) // 64 * 64 + (16 << 20) // 4
+
+
+def test_data_flow_kernel_gives_up_and_recovers(hip, device, oracle):
+    """The give-up path of the data-flow kernel (batch 1, streaming layout, every dependency carried by
+    data): with a limit of one poll, a wave whose x has not arrived gives up at once, the kernel sets
+    *status and every workgroup exits; the same entries on the same workspace with the default limit
+    are then correct twice over, i.e. the halves of the exchange and the launch count were left
+    consistent."""
+    from popxl_addons._gq_hip import GemvSequence, GQHipError
+
+    shapes = [(4096, 4096), (16384, 4096), (4096, 16384), (4096, 4096)]
+    entries, seq, refs, outs = _chained_streaming_case(hip, device, oracle, shapes, seed=71)
+    impatient = GemvSequence(device, spin_limit=1)
+    patient = GemvSequence(device, own_workspace=True)
+    for s2 in (impatient, patient):
+        for i, (x, w, y, ob) in enumerate(entries):
+            s2.add(x, w, None, None, y, ob, wait_previous=i > 0)
+    impatient._finalise()
+    patient._finalise()
+    patient._workspace = impatient._workspace  # the same workspace, one run after the other
+    words = impatient._workspace.view(torch.int32)
+    assert int(words[_FLOW_EPOCH_WORD].item()) == 0
+    impatient.run()
+    torch.cuda.synchronize()
+    assert int(impatient.status.item()) == 1
+    assert int(words[_FLOW_EPOCH_WORD].item()) == 1, "the launch ran on the data-flow kernel and turned the exchange over"
+    with pytest.raises(GQHipError):
+        impatient.check()
+    for run in range(2):
+        for y in outs:
+            y.fill_(float("nan"))
+        patient.run()
+        patient.check()
+        assert int(words[_FLOW_EPOCH_WORD].item()) == run % 2
+        _assert_chain(oracle, seq, refs, outs)
+
+
+def test_gemv_sequence_run_raises_after_a_give_up(hip, device, oracle):
+    """A run that gave up does not pass silently: the next run() of the object raises (it looks at the
+    host copy of the status word that the earlier run left behind), once; after that the object
+    works again."""
+    from popxl_addons._gq_hip import GemvSequence, GQHipError
+
+    shapes = [(4096, 4096), (2048, 4096), (4096, 2048)]
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, 2, chained=True, seed=72)
+    impatient = GemvSequence(device, spin_limit=1)
+    for i, (x, packed, scale, bias, y, ob) in enumerate(seq.keep):
+        impatient.add(x, packed, scale, bias, y, ob, wait_previous=i > 0)
+    impatient.run()
+    torch.cuda.synchronize()
+    assert int(impatient.status.item()) == 1
+    with pytest.raises(GQHipError, match="gave up"):
+        impatient.run()
+    assert int(impatient.status.item()) == 0
+    impatient.spin_limit = 0  # the default limit: the same entries, the same workspace
+    for _ in range(2):
+        for y in outs:
+            y.fill_(float("nan"))
+        impatient.run()
+        impatient.check()
+        _assert_chain(oracle, seq, refs, outs)
+
+
+def test_gemv_sequence_second_stream_is_refused_while_the_first_is_busy(hip, device, oracle):
+    """gq_gemv_sequence_f16 keeps its progress words in a block of the library, per device: a call on
+    another stream while the first stream still has work pending is refused (GQ_ERR_UNSUPPORTED, nothing
+    launched) instead of corrupting both; once the first stream has drained, the other stream may use
+    the block."""
+    from popxl_addons._gq_hip import GQ_ERR_UNSUPPORTED, GQHipError
+
+    shapes = [(4096, 4096), (2048, 4096), (4096, 2048)]
+    seq, refs, outs = _sequence_case(hip, device, oracle, shapes, 2, chained=True, seed=73)
+    other = torch.cuda.Stream(device=device)
+    a = torch.randn((8192, 8192), dtype=torch.float16, device=device)
+    seq.run()  # (the first run copies the entries to the device, which waits for the stream)
+    seq.check()
+    for y in outs:
+        y.fill_(float("nan"))
+    torch.cuda.synchronize()
+    for _ in range(40):  # tens of milliseconds of work on the current stream, then the sequence behind it
+        a @ a
+    seq.run()
+    with torch.cuda.stream(other):
+        with pytest.raises(GQHipError) as refused:
+            seq.run()
+    assert refused.value.code == GQ_ERR_UNSUPPORTED and "another stream" in str(refused.value)
+    seq.check()
+    _assert_chain(oracle, seq, refs, outs)
+    for y in outs:
+        y.fill_(float("nan"))
+    torch.cuda.synchronize()  # (the fills are work of the first stream too)
+    with torch.cuda.stream(other):  # the first stream is idle now
+        seq.run()
+    seq.check()
+    _assert_chain(oracle, seq, refs, outs)
+    seq.run()  # and back, after the other stream has drained
+    seq.check()

@@ -209,3 +209,35 @@ def test_fused_projections_default_layout(hip, device):
         want = torch.cat([layer(x) for layer in layers], dim=-1).float().cpu().numpy()
         got = fused(x).float().cpu().numpy()
         assert normalised_error(got, want) <= 2e-3  # (the K slabs of the two problems differ: other summation order)
+
+
+@pytest.mark.parametrize("dim", [-1, 0])
+def test_layers_on_two_streams_do_not_share_scratch(hip, device, dim):
+    """LinearGQ.build takes its K-split scratch (arrival counters, partial sums) per (device, stream):
+    two layers that run at the same time on different streams give the results they give alone."""
+    from popxl_addons import _gq_hip
+
+    torch.manual_seed(5)
+    layers, xs, want = [], [], []
+    for i in range(2):
+        nn_layer = torch.nn.Linear(4096, 4096, bias=False)
+        layer = LinearGQ(4096, bias=False, group_size=64, dim=dim)
+        variables = layer.init_variables(4096, torch.float16, device)
+        layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=64, dim=dim))
+        layers.append(layer)
+        # (a decode batch for the default layout, 64 rows for dim=0: the shapes whose K is divided through the scratch)
+        xs.append(torch.randn((4 if dim == -1 else 64, 4096), device=device, dtype=torch.float16))
+        want.append(layer(xs[-1]).clone())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=device) for _ in layers]
+    got = [[], []]
+    for _ in range(50):
+        for i, (layer, stream) in enumerate(zip(layers, streams)):
+            with torch.cuda.stream(stream):
+                got[i].append(layer(xs[i]))
+    torch.cuda.synchronize()
+    keys = [k for k in _gq_hip._kn_workspaces if k[1] in {s.cuda_stream for s in streams}]
+    assert len(keys) == 2 and _gq_hip._kn_workspaces[keys[0]].data_ptr() != _gq_hip._kn_workspaces[keys[1]].data_ptr()
+    for i in range(2):
+        for y in got[i]:
+            assert torch.equal(y, want[i])

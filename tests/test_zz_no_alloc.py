@@ -37,12 +37,17 @@ def _with_workspace(hip, device, tensors, k_in, n_out, gs, m_rows, act):
 def _no_alloc(hip, device, tensors, k_in, n_out, gs, m_rows, act):
     x, packed, scale, bias, out_bias = tensors
     y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    import gc
+
+    gc.collect()  # (tensors of earlier tests that are freed during the call would change the figures below)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(device)
+    before, free_before = torch.cuda.memory_allocated(device), torch.cuda.mem_get_info(device)[0]
     hip.call("gq_linear_kn_act_noalloc_f16", x.data_ptr(), m_rows, packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
              out_bias.data_ptr(), y.data_ptr(), n_out, k_in, gs, act, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(device) == before
+    # neither through torch's allocator nor behind its back (device memory as the driver counts it)
+    assert torch.cuda.memory_allocated(device) <= before
+    assert torch.cuda.mem_get_info(device)[0] >= free_before
     return y.cpu().numpy()
 
 
@@ -57,6 +62,52 @@ def test_no_alloc_entry_point_matches_workspace_entry_point(hip, device):
     for _ in range(2):
         for p, (y_want, _) in zip(problems, want):
             assert_bits_equal(_no_alloc(hip, device, *p), y_want, str(p[1:]))
+
+
+def test_no_alloc_entry_point_against_oracle(hip, device, oracle):
+    """Not only equal to its sibling: the no-alloc entry point itself against the oracle's linear over
+    the oracle-decompressed weight (the default layout of LinearGQ at a layer shape of the 6B stack),
+    within the tolerance of the fused paths."""
+    k_in, n_out, gs, m_rows = 4096, 4096, 64, 4
+    tensors = _problem(device, k_in, n_out, gs, m_rows, 300)
+    x, packed, scale, bias, out_bias = (t.cpu().numpy() for t in tensors)
+    w = oracle.np_decompress(packed, scale, bias)  # [k_in, n_out]
+    ref = oracle.np_linear(x, np.ascontiguousarray(w.T), out_bias)
+    for _ in range(2):
+        y = _no_alloc(hip, device, tensors, k_in, n_out, gs, m_rows, 0)
+        err = np.abs(y.astype(np.float64) - ref).max() / np.abs(ref).max()
+        assert err <= 1e-2, err
+
+
+def test_no_alloc_entry_point_refuses_a_second_stream_while_the_first_is_busy(hip, device):
+    """All calls on a GPU share the library's scratch array: a call on another stream while the first
+    stream still has work pending is refused (nothing launched) instead of racing."""
+    from popxl_addons._gq_hip import GQ_ERR_UNSUPPORTED, GQHipError
+
+    k_in, n_out, gs, m_rows = 4096, 4096, 64, 2
+    tensors = _problem(device, k_in, n_out, gs, m_rows, 301)
+    x, packed, scale, bias, out_bias = tensors
+    y = torch.empty((m_rows, n_out), dtype=torch.float16, device=device)
+
+    def call(stream):
+        hip.call("gq_linear_kn_act_noalloc_f16", x.data_ptr(), m_rows, packed.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+                 out_bias.data_ptr(), y.data_ptr(), n_out, k_in, gs, 0, stream.cuda_stream)
+
+    other = torch.cuda.Stream(device=device)
+    a = torch.randn((8192, 8192), dtype=torch.float16, device=device)
+    torch.cuda.synchronize()
+    for _ in range(40):  # tens of milliseconds of work on the current stream
+        a @ a
+    call(torch.cuda.current_stream())
+    with pytest.raises(GQHipError) as refused:
+        call(other)
+    assert refused.value.code == GQ_ERR_UNSUPPORTED and "another stream" in str(refused.value)
+    torch.cuda.synchronize()
+    want = y.clone()
+    y.fill_(float("nan"))
+    call(other)  # the first stream has drained
+    torch.cuda.synchronize()
+    assert torch.equal(want, y)
 
 
 def test_no_alloc_entry_point_rejects_oversized_problems(hip, device):
