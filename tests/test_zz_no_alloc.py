@@ -105,6 +105,7 @@ def test_no_alloc_entry_point_refuses_a_second_stream_while_the_first_is_busy(hi
     torch.cuda.synchronize()
     want = y.clone()
     y.fill_(float("nan"))
+    torch.cuda.synchronize()  # (the copy and the fill are work of the first stream too)
     call(other)  # the first stream has drained
     torch.cuda.synchronize()
     assert torch.equal(want, y)
