@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the 4-bit group-quantization path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decompress|compress|gemv|kn|gemm|stack|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only decompress|compress|gemv|kn|knp|gemm|stack|all]
 
 One "step" is one standalone int4 -> fp16 decompress of the 4096 x 16384 weight (benchmark
 configuration 2: group 64, ~N(0, 0.02) with 0.1 % outliers at +-8 sigma, packed by the
@@ -255,22 +255,26 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     (weight [k_in, n_out], groups along n_out: the default layout of LinearGQ)."""
     import torch
 
-    kn = entry == "gq_linear_kn_act_f16"
+    knp = entry == "gq_linear_knp_act_f16"  # (the same layout, read from its derived copy: the kn streaming layout)
+    kn = entry == "gq_linear_kn_act_f16" or knp
     sets = []
     for s in range(n_sets):
         w = make_weight(k_in, n_out, 200 + s, False, device) if kn else make_weight(n_out, k_in, 200 + s, False, device)
-        sets.append(pack_weight(w))
+        sets.append((hip.prepack_gemv_kn(*pack_weight(w)),) if knp else pack_weight(w))
     g = torch.Generator(device=device)
     g.manual_seed(7)
     x = torch.randn((m_rows, k_in), generator=g, device=device, dtype=torch.float32).to(torch.float16)
     y = torch.empty((m_rows, n_out), dtype=torch.float16, device=device)
     stream = stream_handle()
     with_ws = entry == "gq_linear_act_ws_f16"  # (the layer's entry for the [n_out, k_in] layout: K may be divided over workgroups)
-    ws_bytes = (hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, GROUP) if kn else
+    ws_bytes = (0 if knp else hip.load().gq_linear_kn_workspace_bytes(m_rows, n_out, k_in, GROUP) if kn else
                 hip.load().gq_gemm_workspace_bytes(m_rows, n_out, k_in, GROUP) if with_ws else 0)
     ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=device)
 
     def step(i):
+        if knp:
+            hip.call(entry, x.data_ptr(), m_rows, sets[i % n_sets][0].blob.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP, 0, stream)
+            return
         p, s, b = sets[i % n_sets]
         if kn:
             hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP,
@@ -608,8 +612,10 @@ def headline(result):
             short[key] = {"us": round(extra[key]["us"], 1), "frac": round(extra[key]["hbm_frac"], 3)}
     if "gemv" in extra:  # configuration 3 (+ the stack's third shape): fraction of HBM peak on the packed weight
         short["c3_gemv"] = [_row(r, "hbm_frac") for r in extra["gemv"]]
-    if "linear_kn" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out])
-        short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] <= 16]
+    if "linear_knp" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out]), from the derived copy
+        short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_knp"]]
+    if "linear_kn" in extra:  # ... and from the three variables as they are
+        short["c3_gemv_default_layout_variables"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] <= 16]
         short["gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
     if "gemm" in extra:  # configuration 4: fraction of the dense fp16 MFMA peak
         short["c4_gemm"] = [_row(r, "mfma_frac") for r in extra["gemm"]]
@@ -650,7 +656,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", default="all", choices=["decompress", "compress", "gemv", "kn", "gemm", "stack", "all"])
+    ap.add_argument("--only", default="all", choices=["decompress", "compress", "gemv", "kn", "knp", "gemm", "stack", "all"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stack-modes", default="",
                     help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
@@ -754,6 +760,16 @@ def main():
         extra["linear_kn"].append(r)
         log(f"  kn-layout gemm m=128 [4096->16384]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
         torch.cuda.empty_cache()
+    if args.only in ("kn", "knp", "all"):
+        # ... and from the derived copy that a layer keeps after prepack_for_decode(): the kn streaming layout
+        extra["linear_knp"] = []
+        for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
+            for m in (1, 8):
+                r = bench_linear(hip, device, "gq_linear_knp_act_f16", m, n_out, k_in, 200, 20,
+                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_knp_kernel")
+                extra["linear_knp"].append(r)
+                log(f"  kn streaming layout gemv m={m} [{k_in}->{n_out}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
+                torch.cuda.empty_cache()
     if args.only in ("gemm", "all"):
         extra["gemm"] = []
         for m in (128, 512, 2048):

@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define GQ_ABI_VERSION 2
+#define GQ_ABI_VERSION 3
 
 #define GQ_OK 0
 #define GQ_ERR_NULL_POINTER (-1) /* a required pointer is NULL */
@@ -221,12 +221,12 @@ int gq_linear_kn_act_noalloc_f16(const uint16_t *x, int64_t m_rows, const uint16
  * entry or, at one batch row, of several earlier entries whose y lie end to end in memory (two
  * projections whose results are added, as one entry over the concatenation of their inputs).
  *
- * For group_size 64, k_in % 512 == 0, m_rows <= 4 and 16-byte aligned pointers the whole sequence
- * runs as one persistent kernel (one workgroup per compute unit) that streams the packed weights
- * without a gap between entries; any other sequence runs as one launch per entry.  There are two
- * such kernels: launches of one batch row whose weights are all in the streaming layout (below) and
- * whose entries need nothing but the results they read as x run on the faster of the two; every
- * other launch runs on the general one.  The choice is made per launch of up to 128 entries and
+ * Runs of consecutive entries with group_size 64, k_in % 512 == 0, m_rows <= 4 and 16-byte aligned
+ * pointers execute as one persistent kernel per run of up to 128 entries (one workgroup per compute
+ * unit) that streams the packed weights without a gap between entries; every other entry is a launch
+ * of its own, in stream order.  There are two such kernels: launches of one batch row whose weights are
+ * all in the streaming layout (below) and whose entries need nothing but the results they read as x run
+ * on the faster of the two; every other launch runs on the general one.  The choice is made per launch and
  * changes no result beyond the tolerance of the fused paths.
  *
  *   descs         host copy of the entries (validated here, not read after the call returns)
@@ -266,8 +266,20 @@ typedef struct gq_gemv_desc {
   uint16_t *y;              /* [m_rows, n_out] binary16 */
   int32_t m_rows, n_out, k_in, group_size;
   int32_t wait_entries;     /* entries [0, wait_entries) complete before this one starts */
-  int32_t activation;       /* GQ_ACT_*: epilogue of this entry */
+  int32_t activation;       /* GQ_ACT_*: epilogue of this entry; or-ed with GQ_DESC_KN_LAYOUT for a weight
+                               grouped along the OUTPUT features (below) */
 } gq_gemv_desc;
+
+/*
+ * An entry whose weight is grouped along the output features (LinearGQ with dim = -1 / 1, the
+ * constructor default, popxl_addons/layers/linear_gq.py:26, 59-62): `packed` is the blob written by
+ * gq_gemv_kn_prepack_f16 (below), scale == bias == NULL, group_size 64, n_out % 64 == 0,
+ * k_in % 512 == 0, m_rows <= 16, x and blob 16-byte aligned, y 8-byte.  The entry computes what
+ * gq_linear_knp_act_f16 computes.  Such entries run as a launch of their own inside the sequence
+ * (stream order provides whatever they wait for), next to runs of entries that the persistent
+ * kernels cover.
+ */
+#define GQ_DESC_KN_LAYOUT 0x100
 
 /*
  * Streaming layout of one weight for gq_gemv_sequence_f16.  No counterpart in the reference, whose
@@ -295,6 +307,37 @@ int64_t gq_gemv_sequence_workspace_bytes(void);
 int gq_gemv_sequence_ws_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs_device, int64_t count,
                             int32_t *status, void *workspace, int64_t workspace_bytes, int64_t spin_limit,
                             void *stream);
+
+/*
+ * The default layout of LinearGQ (groups along the OUTPUT features, dim = -1 / 1:
+ * popxl_addons/layers/linear_gq.py:26, 59-62, 99-101) for decode batches, on a derived copy of the
+ * weight.  No counterpart in the reference, whose three variables stay what the rest of the API
+ * takes; this copy is made once when the weights are loaded, like the streaming layout above.
+ *
+ * In the variables a packed word holds 8 consecutive outputs of ONE input feature; a GEMV wants the
+ * codes of an output contiguous along the input features.  With
+ *   y[m][n] = sum_k (x[m][k] scale[k][g]) code[k][n] + sum_k x[m][k] bias[k][g],   g = n / 64,
+ * the scale moves to the activations, so the copy only has to transpose the codes: the KN STREAMING
+ * LAYOUT holds, per group of 64 outputs and chunk of 512 input features, 16 KiB of codes (contiguous
+ * along the input features, in the order the kernel hands them to the matrix instruction) followed by
+ * the group's 512 scales and 512 biases of that chunk: 18432 bytes, the same 0.5625 bytes per weight.
+ * Needs group_size 64, n_out % 64 == 0, k_in % 512 == 0.
+ *
+ *   gq_gemv_kn_prepacked_bytes  size of the blob in bytes, or a negative GQ_ERR_* code
+ *   gq_gemv_kn_prepack_f16      writes the blob (device memory, 16-byte aligned) from the variables
+ *                               packed [k_in, n_out / 64, 16], scale / bias [k_in, n_out / 64] on `stream`
+ *   gq_linear_knp_act_f16       y = act(x w + out_bias) as gq_linear_kn_act_f16 computes it, from the
+ *                               blob, for 1 <= m_rows <= 16 (x, blob 16-byte aligned, y 8-byte); needs no
+ *                               workspace and keeps no state.  The products x scale are rounded to
+ *                               binary16 before they are multiplied with the exact codes; the result is
+ *                               within the tolerance of the fused paths.
+ */
+int64_t gq_gemv_kn_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size);
+int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob,
+                           int64_t n_out, int64_t k_in, int64_t group_size, void *stream);
+int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias,
+                          uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation,
+                          void *stream);
 
 /*
  * Device-side compress for binary16 input: bit-identical packed/scale/bias to

@@ -259,6 +259,29 @@ static int gemv_sequence_common(const gq_gemv_desc *descs, const gq_gemv_desc *d
   for (int64_t i = 0; i < count; ++i) {
     const gq_gemv_desc &d = descs[i];
     const bool blob = d.scale == nullptr && d.bias == nullptr && d.packed != nullptr;
+    if (d.activation & GQ_DESC_KN_LAYOUT) {
+      // a weight grouped along the output features, in the kn streaming layout
+      const int act = d.activation & ~GQ_DESC_KN_LAYOUT;
+      if (!blob)
+        return gq::fail(GQ_ERR_UNSUPPORTED,
+                        "gq_gemv_sequence_f16: entry %lld is marked GQ_DESC_KN_LAYOUT: `packed` must be the blob written by "
+                        "gq_gemv_kn_prepack_f16 and scale, bias NULL", (long long)i);
+      if (!gq::gemv_kn_prepack_shape_ok(d.n_out, d.k_in, d.group_size) || d.m_rows < 1 || d.m_rows > 16)
+        return gq::fail(GQ_ERR_UNSUPPORTED,
+                        "gq_gemv_sequence_f16: entry %lld is in the kn streaming layout, which needs group_size 64, n_out %% 64 == 0, "
+                        "k_in %% 512 == 0 and 1 <= m_rows <= 16 (got group_size=%d n_out=%d k_in=%d m_rows=%d)",
+                        (long long)i, d.group_size, d.n_out, d.k_in, d.m_rows);
+      if (!d.x || !d.y) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_sequence_f16: entry %lld: x or y is NULL", (long long)i);
+      if (gq::misaligned(d.packed, 16) || gq::misaligned(d.x, 16) || gq::misaligned(d.y, 8) || gq::misaligned(d.out_bias, 2))
+        return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_f16: entry %lld: blob and x must be 16-byte aligned, y 8-byte",
+                        (long long)i);
+      if (act < GQ_ACT_NONE || act > GQ_ACT_GELU_TANH)
+        return gq::fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: entry %lld has unknown activation %d", (long long)i, act);
+      if (d.wait_entries < 0 || d.wait_entries > i)
+        return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_sequence_f16: entry %lld has wait_entries=%d outside [0, %lld]",
+                        (long long)i, d.wait_entries, (long long)i);
+      continue;
+    }
     if (blob) {
       // the weight in the streaming layout: only the persistent kernel reads it
       if (d.group_size != 64 || d.k_in <= 0 || d.k_in % 512 != 0 || d.m_rows < 1 || d.m_rows > 4 || d.n_out < 1)
@@ -330,6 +353,50 @@ int gq_gemv_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uin
   if (gq::misaligned(packed, 16) || gq::misaligned(scale, 16) || gq::misaligned(bias, 16) || gq::misaligned(blob, 16))
     return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_prepack_f16: pointers must be 16-byte aligned");
   return gq::launch_gemv_prepack(packed, scale, bias, blob, n_out, k_in, (hipStream_t)stream);
+}
+
+int64_t gq_gemv_kn_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size) {
+  if (n_out < 0 || k_in < 0) return gq::fail(GQ_ERR_BAD_SHAPE, "gq_gemv_kn_prepacked_bytes: negative size");
+  if (n_out == 0 || k_in == 0) return 0;
+  if (!gq::gemv_kn_prepack_shape_ok(n_out, k_in, group_size))
+    return gq::fail(GQ_ERR_UNSUPPORTED,
+                    "gq_gemv_kn_prepacked_bytes: the kn streaming layout needs group_size 64, n_out %% 64 == 0, k_in %% 512 == 0, "
+                    "n_out <= 2^22 and k_in <= 2^24 (got group_size=%lld n_out=%lld k_in=%lld)",
+                    (long long)group_size, (long long)n_out, (long long)k_in);
+  return gq::gemv_kn_prepacked_bytes(n_out, k_in);
+}
+
+int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
+                           int64_t k_in, int64_t group_size, void *stream) {
+  const int64_t bytes = gq_gemv_kn_prepacked_bytes(n_out, k_in, group_size);
+  if (bytes < 0) return (int)bytes;
+  if (bytes == 0) return GQ_OK;
+  if (!packed || !scale || !bias || !blob) return gq::fail(GQ_ERR_NULL_POINTER, "gq_gemv_kn_prepack_f16: NULL pointer argument");
+  if (gq::misaligned(packed, 2) || gq::misaligned(scale, 2) || gq::misaligned(bias, 2) || gq::misaligned(blob, 16))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_kn_prepack_f16: the blob must be 16-byte aligned, the other pointers 2-byte");
+  return gq::launch_gemv_kn_prepack(packed, scale, bias, blob, n_out, k_in, (hipStream_t)stream);
+}
+
+int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y,
+                          int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation, void *stream) {
+  if (m_rows < 0 || n_out < 0 || k_in < 0)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_knp_act_f16: negative size (m_rows=%lld n_out=%lld k_in=%lld)", (long long)m_rows,
+                    (long long)n_out, (long long)k_in);
+  if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: unknown activation %d", (int)activation);
+  if (m_rows == 0 || n_out == 0) return GQ_OK;
+  if (m_rows > 16)
+    return gq::fail(GQ_ERR_UNSUPPORTED,
+                    "gq_linear_knp_act_f16: m_rows=%lld exceeds 16: the kn streaming layout serves decode batches; larger batches "
+                    "go through gq_linear_kn_act_f16 on the three variables", (long long)m_rows);
+  if (!gq::gemv_kn_prepack_shape_ok(n_out, k_in, group_size))
+    return gq::fail(GQ_ERR_UNSUPPORTED,
+                    "gq_linear_knp_act_f16: the kn streaming layout needs group_size 64, n_out %% 64 == 0 and k_in %% 512 == 0 (got "
+                    "group_size=%lld n_out=%lld k_in=%lld)", (long long)group_size, (long long)n_out, (long long)k_in);
+  if (!x || !blob || !y) return gq::fail(GQ_ERR_NULL_POINTER, "gq_linear_knp_act_f16: x, blob and y must not be NULL");
+  if (gq::misaligned(x, 16) || gq::misaligned(blob, 16) || gq::misaligned(y, 8) || gq::misaligned(out_bias, 2))
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_knp_act_f16: x and blob must be 16-byte aligned, y 8-byte, out_bias 2-byte");
+  return gq::launch_gemv_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
 }
 
 int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,

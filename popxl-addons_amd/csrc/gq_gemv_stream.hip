@@ -1016,50 +1016,44 @@ void plan_launch(const gq_gemv_desc *e, int n, int64_t first, bool any_fit, int 
 
 }  // namespace
 
-// launches of weights in the streaming layout whose dependencies all travel through the exchange
-// run on the data-flow kernel of gq_gemv_flow.hip
-
 int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, int64_t count, int *status,
                          void *workspace, int64_t spin_limit, hipStream_t stream) {
-  int max_m = 1;
-  bool supported = count <= (1 << 20);
-  for (int64_t i = 0; i < count && supported; ++i) {
-    if (host[i].m_rows > max_m) max_m = host[i].m_rows;
-    supported = stream_shape_ok(host[i]);
-  }
-  if (!supported) {
-    // any other shape: one launch per entry; stream order provides every dependency
-    for (int64_t i = 0; i < count; ++i)
-      if (prepacked(host[i]))
-        return fail(GQ_ERR_UNSUPPORTED,
-                    "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which only the persistent kernel "
-                    "reads, but the sequence holds a shape outside it (group 64, k_in %% 512 == 0, m_rows <= 4, 16-byte "
-                    "aligned)", (long long)i);
-    for (int64_t i = 0; i < count; ++i) {
-      const gq_gemv_desc &d = host[i];
-      const int rc = launch_gemv(d.x, d.m_rows, d.packed, d.scale, d.bias, d.out_bias, d.y, d.n_out, d.k_in,
-                                 d.group_size, d.activation, stream);
-      if (rc != GQ_OK) return rc;
+  if (count > (1 << 20)) return fail(GQ_ERR_UNSUPPORTED, "gq_gemv_sequence_f16: more than 2^20 entries");
+  // Runs of consecutive entries that the persistent kernels cover (group 64, k_in % 512 == 0, m_rows <= 4,
+  // 16-byte aligned, groups along the input features) go to them, up to kMaxEntries per launch; every
+  // other entry is a launch of its own.  Launches execute in stream order, so whatever an entry
+  // waits for in an earlier launch is complete when it starts.
+  auto persistent = [&](int64_t i) { return !(host[i].activation & GQ_DESC_KN_LAYOUT) && stream_shape_ok(host[i]); };
+  bool any_persistent = false;
+  for (int64_t i = 0; i < count; ++i) {
+    if (persistent(i)) {
+      any_persistent = true;
+    } else if (prepacked(host[i]) && !(host[i].activation & GQ_DESC_KN_LAYOUT)) {
+      return fail(GQ_ERR_UNSUPPORTED,
+                  "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which only the persistent kernel "
+                  "reads, but its shape is outside that kernel (group 64, k_in %% 512 == 0, m_rows <= 4, 16-byte aligned)",
+                  (long long)i);
     }
-    return GQ_OK;
   }
-  int dev = 0;
-  const int grid = stream_grid(&dev);
-  if (grid == 0) return GQ_ERR_NO_DEVICE;
+  int dev = 0, grid = 0;
   unsigned *words = static_cast<unsigned *>(workspace);
-  if (!words) {
-    // the library's own block of this device (its address differs from device to device)
-    static SharedBlockGuard guard = {};
-    const int claimed = claim_shared_block(guard, dev, stream, "gq_gemv_sequence_f16");
-    if (claimed != GQ_OK) return claimed;
-    static unsigned *own[kMaxDevices] = {nullptr};
-    if (!own[dev]) {
-      void *ptr = nullptr;
-      const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sequence_words));
-      if (e != hipSuccess || !ptr) return fail((int)e, "hipGetSymbolAddress(progress words): %s", hipGetErrorString(e));
-      own[dev] = static_cast<unsigned *>(ptr);
+  if (any_persistent) {
+    grid = stream_grid(&dev);
+    if (grid == 0) return GQ_ERR_NO_DEVICE;
+    if (!words) {
+      // the library's own block of this device (its address differs from device to device)
+      static SharedBlockGuard guard = {};
+      const int claimed = claim_shared_block(guard, dev, stream, "gq_gemv_sequence_f16");
+      if (claimed != GQ_OK) return claimed;
+      static unsigned *own[kMaxDevices] = {nullptr};
+      if (!own[dev]) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_sequence_words));
+        if (e != hipSuccess || !ptr) return fail((int)e, "hipGetSymbolAddress(progress words): %s", hipGetErrorString(e));
+        own[dev] = static_cast<unsigned *>(ptr);
+      }
+      words = own[dev];
     }
-    words = own[dev];
   }
   const unsigned spins = spin_limit > 0 ? (unsigned)(spin_limit < 0x7fffffff ? spin_limit : 0x7fffffff) : kDefaultSpinLimit;
 #define GQ_STREAM(MC, NS)                                                                                     \
@@ -1074,23 +1068,44 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
       if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));              \
       configured[dev] = true;                                                                                 \
     }                                                                                                         \
-    for (int64_t first = 0; first < count; first += kMaxEntries) {                                            \
-      const int n = (int)(count - first < kMaxEntries ? count - first : kMaxEntries);                         \
-      SequencePlan plan;                                                                                      \
-      plan_launch(host + first, n, first, true, grid, plan);                                                  \
-      if (flow_eligible(host + first, n, plan)) {                                                             \
-        const int rc = launch_flow(host + first, device + first, n, status, words, spins, plan, grid, dev, stream); \
-        if (rc != GQ_OK) return rc;                                                                           \
-        continue;                                                                                             \
-      }                                                                                                       \
-      plan_launch(host + first, n, first, false, grid, plan);                                                 \
-      kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status, words, spins, plan); \
-    }                                                                                                         \
+    kern<<<dim3(grid), dim3(kThreadsAll), lds_bytes, stream>>>(device + first, n, status, words, spins, plan); \
   } while (0)
-  if (max_m <= 2) GQ_STREAM(2, 3);
-  else GQ_STREAM(4, 3);
+  int64_t first = 0;
+  while (first < count) {
+    if (!persistent(first)) {
+      const gq_gemv_desc &d = host[first];
+      const int act = d.activation & ~GQ_DESC_KN_LAYOUT;
+      const int rc = (d.activation & GQ_DESC_KN_LAYOUT)
+                         ? launch_gemv_knp(d.x, d.m_rows, d.packed, d.out_bias, d.y, d.n_out, d.k_in, act, stream)
+                         : launch_gemv(d.x, d.m_rows, d.packed, d.scale, d.bias, d.out_bias, d.y, d.n_out, d.k_in,
+                                       d.group_size, act, stream);
+      if (rc != GQ_OK) return rc;
+      ++first;
+      continue;
+    }
+    int n = 0, max_m = 1;
+    while (n < kMaxEntries && first + n < count && persistent(first + n)) {
+      if (host[first + n].m_rows > max_m) max_m = host[first + n].m_rows;
+      ++n;
+    }
+    SequencePlan plan;
+    // launches of weights in the streaming layout whose dependencies all travel through the exchange
+    // run on the data-flow kernel of gq_gemv_flow.hip
+    plan_launch(host + first, n, first, true, grid, plan);
+    if (flow_eligible(host + first, n, plan)) {
+      const int rc = launch_flow(host + first, device + first, n, status, words, spins, plan, grid, dev, stream);
+      if (rc != GQ_OK) return rc;
+    } else {
+      plan_launch(host + first, n, first, false, grid, plan);
+      if (max_m <= 2) GQ_STREAM(2, 3);
+      else GQ_STREAM(4, 3);
+      const int rc = check_launch("gemv_stream_kernel");
+      if (rc != GQ_OK) return rc;
+    }
+    first += n;
+  }
 #undef GQ_STREAM
-  return check_launch("gemv_stream_kernel");
+  return GQ_OK;
 }
 
 // ---- the streaming layout: block (rb, c) = what the ring slot of work item (rb, c) holds

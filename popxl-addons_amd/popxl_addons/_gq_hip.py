@@ -10,13 +10,14 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _DEFAULT_LIB = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libgq_hip.so")
 
-GQ_ABI_VERSION = 2
+GQ_ABI_VERSION = 3
 GQ_ERR_NULL_POINTER = -1
 GQ_ERR_BAD_SHAPE = -2
 GQ_ERR_MISALIGNED = -3
 GQ_ERR_UNSUPPORTED = -4
 GQ_ERR_NO_DEVICE = -5
 GQ_ACT_NONE, GQ_ACT_RELU, GQ_ACT_GELU_TANH = 0, 1, 2
+GQ_DESC_KN_LAYOUT = 0x100  # or-ed into a sequence entry's activation: weight grouped along the output features
 ACTIVATIONS = {None: GQ_ACT_NONE, "none": GQ_ACT_NONE, "relu": GQ_ACT_RELU, "gelu_tanh": GQ_ACT_GELU_TANH}
 
 
@@ -49,6 +50,9 @@ EXPORTS = (
     "gq_gemv_sequence_ws_f16",
     "gq_gemv_prepacked_bytes",
     "gq_gemv_prepack_f16",
+    "gq_gemv_kn_prepacked_bytes",
+    "gq_gemv_kn_prepack_f16",
+    "gq_linear_knp_act_f16",
     "gq_compress_f16",
     "gq_compress_f32",
 )
@@ -117,6 +121,12 @@ def load():
     lib.gq_gemv_prepacked_bytes.restype = i64
     lib.gq_gemv_prepack_f16.argtypes = [p, p, p, p, i64, i64, i64, p]
     lib.gq_gemv_prepack_f16.restype = ctypes.c_int
+    lib.gq_gemv_kn_prepacked_bytes.argtypes = [i64, i64, i64]
+    lib.gq_gemv_kn_prepacked_bytes.restype = i64
+    lib.gq_gemv_kn_prepack_f16.argtypes = [p, p, p, p, i64, i64, i64, p]
+    lib.gq_gemv_kn_prepack_f16.restype = ctypes.c_int
+    lib.gq_linear_knp_act_f16.argtypes = [p, i64, p, p, p, i64, i64, i64, ctypes.c_int32, p]
+    lib.gq_linear_knp_act_f16.restype = ctypes.c_int
     for name in ("gq_compress_f16", "gq_compress_f32"):
         fn = getattr(lib, name)
         fn.argtypes = [p, p, p, p, p, i64, i64, i64, p]
@@ -164,11 +174,13 @@ def linear_kn_workspace(device, nbytes):
 
 
 class PrepackedWeight:
-    """One weight in the streaming layout of gq_gemv_prepack_f16 (a device blob that only
-    GemvSequence entries read); made from the three LinearGQ variables by prepack_gemv()."""
+    """One weight in a streaming layout: a device blob derived from the three LinearGQ variables.
+    layout "nk": groups along the input features (LinearGQ dim=0), made by prepack_gemv(), read by
+    GemvSequence entries only; layout "kn": groups along the output features (dim=-1 / 1, the
+    default), made by prepack_gemv_kn(), read by GemvSequence entries and by linear_knp()."""
 
-    def __init__(self, blob, n_out, k_in, group_size):
-        self.blob, self.n_out, self.k_in, self.group_size = blob, n_out, k_in, group_size
+    def __init__(self, blob, n_out, k_in, group_size, layout="nk"):
+        self.blob, self.n_out, self.k_in, self.group_size, self.layout = blob, n_out, k_in, group_size, layout
 
 
 def prepack_gemv(packed, scale, bias):
@@ -188,6 +200,42 @@ def prepack_gemv(packed, scale, bias):
         call("gq_gemv_prepack_f16", packed.data_ptr(), scale.data_ptr(), bias.data_ptr(), blob.data_ptr(), n_out, k_in,
              group_size, torch.cuda.current_stream(packed.device).cuda_stream)
     return PrepackedWeight(blob, n_out, k_in, group_size)
+
+
+def prepack_gemv_kn(packed, scale, bias):
+    """The variables of a layer grouped along the OUTPUT features -- packed uint16 [k_in, n_out / 64, 16],
+    scale / bias float16 [k_in, n_out / 64, 1] on the GPU -> PrepackedWeight in the kn streaming layout."""
+    import torch
+
+    k_in, n_groups, n_ids = packed.shape
+    n_out, group_size = n_groups * n_ids * 4, n_ids * 4
+    for t in (packed, scale, bias):
+        assert t.is_cuda and t.is_contiguous()
+    lib = load()
+    nbytes = lib.gq_gemv_kn_prepacked_bytes(n_out, k_in, group_size)
+    if nbytes < 0:
+        raise GQHipError("gq_gemv_kn_prepacked_bytes", nbytes, lib.gq_last_error().decode("utf-8", "replace"))
+    with torch.cuda.device(packed.device):
+        blob = torch.empty(nbytes, dtype=torch.uint8, device=packed.device)
+        call("gq_gemv_kn_prepack_f16", packed.data_ptr(), scale.data_ptr(), bias.data_ptr(), blob.data_ptr(), n_out, k_in,
+             group_size, torch.cuda.current_stream(packed.device).cuda_stream)
+    return PrepackedWeight(blob, n_out, k_in, group_size, layout="kn")
+
+
+def linear_knp(x, weight, out_bias=None, activation=None, y=None):
+    """y = act(x @ w + out_bias) for x float16 [m_rows <= 16, k_in] on the GPU and a PrepackedWeight in
+    the kn streaming layout (gq_linear_knp_act_f16)."""
+    import torch
+
+    assert weight.layout == "kn" and x.is_cuda and x.is_contiguous() and x.shape[-1] == weight.k_in
+    m_rows = x.shape[0]
+    with torch.cuda.device(x.device):
+        if y is None:
+            y = torch.empty((m_rows, weight.n_out), dtype=torch.float16, device=x.device)
+        call("gq_linear_knp_act_f16", x.data_ptr(), m_rows, weight.blob.data_ptr(), 0 if out_bias is None else out_bias.data_ptr(),
+             y.data_ptr(), weight.n_out, weight.k_in, weight.group_size, activation_code(activation),
+             torch.cuda.current_stream(x.device).cuda_stream)
+    return y
 
 
 class GemvSequence:
@@ -235,13 +283,15 @@ class GemvSequence:
         self._status_event = None  # recorded behind that copy; None: no copy under way
 
     def add(self, x, packed, scale, bias, y, out_bias=None, wait_previous=False, wait_for=None, activation=None):
-        """`packed` may be a PrepackedWeight (then scale and bias are None)."""
+        """`packed` may be a PrepackedWeight of either layout (then scale and bias are None)."""
         m_rows, k_in = x.shape
+        layout_flag = 0
         if isinstance(packed, PrepackedWeight):
             assert scale is None and bias is None and packed.k_in == k_in
             n_out, group_size = packed.n_out, packed.group_size
             pointers = (packed.blob.data_ptr(), 0, 0)
             tensors = (x, packed.blob, y)
+            layout_flag = GQ_DESC_KN_LAYOUT if packed.layout == "kn" else 0
         else:
             n_out, n_groups, n_ids = packed.shape
             assert n_groups * n_ids * 4 == k_in
@@ -258,7 +308,7 @@ class GemvSequence:
         self.entries.append(
             (x.data_ptr(), *pointers,
              0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), m_rows, n_out, k_in, group_size,
-             wait_entries, activation_code(activation))
+             wait_entries, activation_code(activation) | layout_flag)
         )
         self.keep.append((x, packed, scale, bias, y, out_bias))
         self._host = None

@@ -55,6 +55,7 @@ class LinearGQ:
         self.group_size = group_size
         self.dim = dim
         self.variables: Optional[NamedTensors] = None
+        self._decode_copy = None  # dim=-1 / 1 only: the weight in the kn streaming layout (prepack_for_decode)
 
     # ----------------------------------------------------------------------------- variables
 
@@ -97,6 +98,9 @@ class LinearGQ:
             weights = weights(self.variables)
         for var, value in weights.items():
             var.data.copy_(torch.from_numpy(np.ascontiguousarray(value)).to(var.data.device))
+        if self._decode_copy is not None:  # (a derived copy of the variables: make it again)
+            self._decode_copy = None
+            self.prepack_for_decode()
 
     # --------------------------------------------------------------------------------- build
 
@@ -146,6 +150,9 @@ class LinearGQ:
                 ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None
                 _gq_hip.call("gq_linear_act_ws_f16", *args, 0 if ws is None else ws.data_ptr(),
                              0 if ws is None else ws.numel(), stream)
+            elif m_rows <= 16 and self._decode_copy is not None:
+                # groups along the output features, decode batch, the derived copy is there
+                _gq_hip.linear_knp(x2, self._decode_copy, b, act, y)
             else:
                 # groups along the output features: weight rows are input features
                 need = _gq_hip.load().gq_linear_kn_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)
@@ -229,15 +236,28 @@ class LinearGQ:
 
     def prepacked(self):
         """The weight in the streaming layout that `_gq_hip.GemvSequence.add` accepts in place of the
-        three variables (a device copy made by gq_gemv_prepack_f16; dim=0, group_size 64 and input
-        features a multiple of 512 only).  The layer keeps its variables; make the copy again after
-        `load_weights`."""
-        if self.dim != 0:
-            raise NotImplementedError("LinearGQ.prepacked: only dim=0 layers feed the GEMV sequence kernel")
+        three variables: a device copy of the same 0.5625 bytes per weight, made by
+        gq_gemv_prepack_f16 (dim=0: group_size 64, input features a multiple of 512) or
+        gq_gemv_kn_prepack_f16 (dim=-1 / 1, the default: group_size 64, input features a multiple of
+        512; the output features are a multiple of 64 by construction).  The layer keeps its variables;
+        make the copy again after `load_weights`."""
         if self.variables is None:
             raise ValueError("LinearGQ.prepacked: the layer has no variables yet (build it or call init_variables)")
         v = self.variables
-        return _gq_hip.prepack_gemv(v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data)
+        make = _gq_hip.prepack_gemv if self.dim == 0 else _gq_hip.prepack_gemv_kn
+        return make(v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data)
+
+    def prepack_for_decode(self):
+        """dim=-1 / 1 (the default layout): keep a copy of the weight in the kn streaming layout, from
+        which `build` then serves batches of up to 16 rows (gq_linear_knp_act_f16: about twice as fast
+        as the kernel that reads the variables, at the price of a second copy of the packed weight);
+        larger batches still read the variables.  `load_weights` renews the copy.  Returns the copy
+        (a `_gq_hip.PrepackedWeight`, which `GemvSequence.add` accepts).  For dim=0 nothing is kept:
+        the variables themselves are what the decode kernel reads."""
+        if self.dim == 0:
+            return self.prepacked()
+        self._decode_copy = self.prepacked()
+        return self._decode_copy
 
     # ------------------------------------------------------------------------- weight mapping
 

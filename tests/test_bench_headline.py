@@ -39,9 +39,10 @@ def full_detail():
         "gpu_equals_cpu_baseline_bits": True,
         "decompress_transposed": {"rows": 4096, "cols": 16384, "us": 26.3456789, "gbs": 6531.123456, "hbm_frac": 0.81612345,
                                   "roofline": bench.hbm_roofline("decompress_transposed_tile_kernel", 171966464.0, 0.0263)},
-        "gemv": [_linear_row(m, n, k, "gemv_mfma_kernel / gemv_stream_single_kernel", "hbm") for n, k in shapes for m in (1, 8, 16)],
-        "linear_kn": [_linear_row(m, n, k, "gemv_kn_kernel", "hbm") for n, k in shapes for m in (1, 8, 16)]
+        "gemv": [_linear_row(m, n, k, "gemv_mfma_kernel / gemv_stream_single_kernel", "hbm") for n, k in shapes for m in (1, 8)],
+        "linear_kn": [_linear_row(m, n, k, "gemv_kn_kernel", "hbm") for n, k in shapes for m in (1, 8)]
         + [_linear_row(128, 16384, 4096, "gemm_kn_tile_kernel", "mfma")],
+        "linear_knp": [_linear_row(m, n, k, "gemv_knp_kernel", "hbm") for n, k in shapes for m in (1, 8)],
         "gemm": [_linear_row(m, 16384, 4096, "gemm_pipe2_kernel", "mfma") for m in (128, 512, 2048)],
         "gemm_other_shapes": [_linear_row(512, 4096, 4096, "gemm_pipe2_kernel", "mfma") for _ in range(7)],
         "stack": [_stack(m) for m in (1, 4, 8, 16)],
@@ -86,7 +87,8 @@ def test_headline_is_short_and_complete():
         assert back["cpu_baseline"][key] == detail["cpu_baseline"][key]
     assert "legs" not in back["cpu_baseline"]
     # one short record per benchmark shape of configurations 3, 4 and 5
-    assert len(back["extra"]["c3_gemv"]) == 9 and len(back["extra"]["c3_gemv_default_layout"]) == 9
+    assert len(back["extra"]["c3_gemv"]) == 6 and len(back["extra"]["c3_gemv_default_layout"]) == 6
+    assert len(back["extra"]["c3_gemv_default_layout_variables"]) == 6
     assert [r["m"] for r in back["extra"]["c4_gemm"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c5_stack"]] == [1, 4, 8, 16]
     for r in back["extra"]["c5_stack"]:
