@@ -37,35 +37,42 @@ constexpr int kKnUnitBytes = 18432;
 constexpr int kKnWaves = 8;
 
 // 8 codes of a word of the kn streaming layout as fp16, in the order of their input features:
-// (64 + c, 64 + c, 1024 + c, 1024 + c) twice.  5 VALU instructions.
+// (64 + c, 64 + c, 1024 + c, 1024 + c) twice.  5 VALU instructions: the masks and magic numbers come
+// in vector registers that the compiler cannot see through, which makes it select v_and_or_b32.
+// (Plain C, not inline assembly: a VALU write to a register that an MFMA in flight still reads or is
+// going to write needs wait states, and the compiler's hazard recogniser does not look into assembly
+// -- with the results wrong now and then, whenever the register allocator re-used such a register.)
 __device__ __forceinline__ half8_t kn_raw_codes(uint32_t w, uint32_t mask_lo, uint32_t mask_hi, uint32_t magic_lo,
                                                 uint32_t magic_hi) {
   const uint32_t hi = w >> 8;
   uint4_t v;
-  v.x = and_or(hi, mask_hi, magic_hi);  // nibbles 3, 7: features 0, 1
-  v.y = and_or(hi, mask_lo, magic_lo);  // nibbles 2, 6: features 2, 3
-  v.z = and_or(w, mask_hi, magic_hi);   // nibbles 1, 5: features 4, 5
-  v.w = and_or(w, mask_lo, magic_lo);   // nibbles 0, 4: features 6, 7
+  v.x = (hi & mask_hi) | magic_hi;  // nibbles 3, 7: features 0, 1
+  v.y = (hi & mask_lo) | magic_lo;  // nibbles 2, 6: features 2, 3
+  v.z = (w & mask_hi) | magic_hi;   // nibbles 1, 5: features 4, 5
+  v.w = (w & mask_lo) | magic_lo;   // nibbles 0, 4: features 6, 7
   return __builtin_bit_cast(half8_t, v);
 }
 
 // Sums of N values per lane over the 64 lanes of a wave: each exchange halves the values a lane
 // keeps (the lane with the exchanged bit clear keeps the lower half), then the lanes that hold the
 // same value add up.  Afterwards lane l holds the sum of value l / (64 / N) in v[0].
-template <int N>
+template <int N, int WIDTH = 32>
 __device__ __forceinline__ void wave_sums(float (&v)[N], int lane) {
-  int width = 32;
+  if constexpr (N > 1) {
+    const bool upper = (lane & WIDTH) != 0;
+    float kept[N / 2];
 #pragma unroll
-  for (int n = N; n > 1; n >>= 1, width >>= 1) {
-    const bool upper = (lane & width) != 0;
-#pragma unroll
-    for (int i = 0; i < n / 2; ++i) {
-      const float send = upper ? v[i] : v[i + n / 2];
-      const float keep = upper ? v[i + n / 2] : v[i];
-      v[i] = keep + __shfl_xor(send, width, 64);
+    for (int i = 0; i < N / 2; ++i) {
+      const float send = upper ? v[i] : v[i + N / 2];
+      const float keep = upper ? v[i + N / 2] : v[i];
+      kept[i] = keep + __shfl_xor(send, WIDTH, 64);
     }
+    wave_sums<N / 2, WIDTH / 2>(kept, lane);
+    v[0] = kept[0];
+  } else {
+#pragma unroll
+    for (int width = WIDTH; width > 0; width >>= 1) v[0] += __shfl_xor(v[0], width, 64);
   }
-  for (; width > 0; width >>= 1) v[0] += __shfl_xor(v[0], width, 64);
 }
 
 constexpr int knp_region_bytes(int r, int xm) { return (xm > r ? xm : r) * 1024; }
@@ -110,60 +117,91 @@ __global__ __launch_bounds__(kKnWaves * 64) void gemv_knp_kernel(const half_t *_
   const char *const gbase = blob + (int64_t)group * n_chunks * kKnUnitBytes + lane * 16;
 
   uint32_t kMaskLo = 0x000F000Fu, kMaskHi = 0x00F000F0u, kMagicLo = 0x64006400u, kMagicHi = 0x54005400u;
+  asm volatile("" : "+v"(kMaskLo), "+v"(kMaskHi), "+v"(kMagicLo), "+v"(kMagicHi));
   const half2_t kNeg64 = {(half_t)-64.f, (half_t)-64.f}, kNeg1024 = {(half_t)-1024.f, (half_t)-1024.f};
 
   float4_t acc[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-  float cacc[XM];  // this lane's share of  sum_k x bias - sum_k off xs  per batch row
+  float cbias[XM], coff[XM];  // this lane's share of  sum_k x bias  and of  - sum_k off xs  per batch row
 #pragma unroll
-  for (int m = 0; m < XM; ++m) cacc[m] = 0.f;
+  for (int m = 0; m < XM; ++m) cbias[m] = coff[m] = 0.f;
 
   char *const stage = region[wave];
   const int x_row = r < m_rows ? r : 0;  // (columns past the batch are never stored: they may hold any row)
-  for (int c = wave; c < n_chunks; c += kKnWaves) {
+  // (batch rows past m_rows: the last row again -- no branches in the loop; their products are never read)
+  const char *const x_lane = reinterpret_cast<const char *>(x) + lane * 16;
+
+  struct Chunk {  // what a wave loads of one chunk
+    uint4_t sv, bv, xq[XM], wq[4][R];
+  };
+  // What the scaled activations need first, then the codes in the order of their use: loads land in
+  // the order issued.
+  auto issue = [&](Chunk &k, int c) {
     const char *const u = gbase + (int64_t)c * kKnUnitBytes;
-    uint4_t wq[R][4];
+    k.sv = *reinterpret_cast<const uint4_t *>(u + 16384);
+    k.bv = *reinterpret_cast<const uint4_t *>(u + 17408);
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-#pragma unroll
-      for (int s = 0; s < 4; ++s) wq[i][s] = *reinterpret_cast<const uint4_t *>(u + (j0 + i) * 4096 + s * 1024);
-    const uint4_t sv = *reinterpret_cast<const uint4_t *>(u + 16384);
-    const uint4_t bv = *reinterpret_cast<const uint4_t *>(u + 17408);
-    uint4_t xq[XM];
-#pragma unroll
-    for (int m = 0; m < XM; ++m) {
-      xq[m] = uint4_t{0u, 0u, 0u, 0u};
-      if (m < m_rows) xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + c * 512 + lane * 8);
-    }
-    // ---- x times scale into the stage; the sums that take out the offsets and bring in the bias
-#pragma unroll
-    for (int m = 0; m < XM; ++m) {
-      if (m < m_rows) {
-        uint4_t xs;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const half2_t xv = as_half2(xq[m][t]);
-          const half2_t p = xv * as_half2(sv[t]);  // (one rounding: the value the MFMA multiplies)
-          xs[t] = __builtin_bit_cast(uint32_t, p);
-          cacc[m] = __builtin_amdgcn_fdot2(xv, as_half2(bv[t]), cacc[m], false);
-          cacc[m] = __builtin_amdgcn_fdot2(p, (t & 1) ? kNeg1024 : kNeg64, cacc[m], false);
-        }
-        *reinterpret_cast<uint4_t *>(stage + m * 1024 + ((lane ^ m) & 63) * 16) = xs;
-      }
-    }
-    // ---- expand and multiply
+    for (int m = 0; m < XM; ++m)
+      k.xq[m] = *reinterpret_cast<const uint4_t *>(x_lane + ((int64_t)min(m, m_rows - 1) * k_in + c * 512) * 2);
 #pragma unroll
     for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < R; ++i) k.wq[s][i] = *reinterpret_cast<const uint4_t *>(u + (j0 + i) * 4096 + s * 1024);
+  };
+  // The empty assembly statements pin the order: every load in front of the first of them is issued
+  // before it (left to itself the compiler moves loads down to their first use, between the MFMAs,
+  // or an instruction that needs the first load up between the loads: either way a memory latency
+  // is waited out with most of the chunk not yet requested), and a loaded value is only touched
+  // behind its own statement, i.e. when the loads in front of it have landed.
+  auto work = [&](Chunk &k) {
+    asm volatile("" : "+v"(k.sv), "+v"(k.bv) : : "memory");
+    // ---- x times scale into the stage; the sums that take out the offsets and bring in the bias
+    // (two sums per batch row and dot products of all rows in turn: no long chains of dependent instructions)
+#pragma unroll
+    for (int m = 0; m < XM; ++m) asm volatile("" : "+v"(k.xq[m]));
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+      for (int m = 0; m < XM; ++m) {
+        const half2_t xv = as_half2(k.xq[m][t]);
+        const half2_t p = xv * as_half2(k.sv[t]);  // (one rounding: the value the MFMA multiplies)
+        k.xq[m][t] = __builtin_bit_cast(uint32_t, p);
+        cbias[m] = __builtin_amdgcn_fdot2(xv, as_half2(k.bv[t]), cbias[m], false);
+        coff[m] = __builtin_amdgcn_fdot2(p, (t & 1) ? kNeg1024 : kNeg64, coff[m], false);
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < XM; ++m) *reinterpret_cast<uint4_t *>(stage + m * 1024 + ((lane ^ m) & 63) * 16) = k.xq[m];
+    // ---- expand and multiply
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+#pragma unroll
+      for (int i = 0; i < R; ++i) asm volatile("" : "+v"(k.wq[s][i]));
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const half8_t b = *reinterpret_cast<const half8_t *>(stage + x_row * 1024 + ((s * 16 + kc * 4 + w) ^ x_row) * 16);
 #pragma unroll
         for (int i = 0; i < R; ++i)
-          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kn_raw_codes(wq[i][s][w], kMaskLo, kMaskHi, kMagicLo, kMagicHi), b,
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kn_raw_codes(k.wq[s][i][w], kMaskLo, kMaskHi, kMagicLo, kMagicHi), b,
                                                           acc[i], 0, 0, 0);
+        // (four row blocks and many batch rows: the expanded codes of later steps would not fit the registers)
+        if (R * XM >= 32) __builtin_amdgcn_sched_barrier(0);
       }
+    }
+  };
+  // (Requesting a wave's next chunk before it works on the current one -- two chunks' worth of
+  // registers -- was measured and is slower: 16384 -> 4096 at one batch row 10.0 against 9.7 us, at eight
+  // rows, where the registers no longer suffice, 17.6 against 14.7 us.  The other waves of the
+  // compute unit keep the memory system busy while one of them computes.)
+  for (int c = wave; c < n_chunks; c += kKnWaves) {
+    Chunk a;
+    issue(a, c);
+    work(a);
   }
+  float cacc[XM];
+#pragma unroll
+  for (int m = 0; m < XM; ++m) cacc[m] = cbias[m] + coff[m];
   // ---- the wave's sums: the per-lane corrections over its 64 lanes, then everything into LDS
   wave_sums<XM>(cacc, lane);
   if (lane < 16) corr[wave][lane] = 0.f;
@@ -272,8 +310,9 @@ int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const u
     const double bytes = (double)n_out * k_in * 0.5 + 0.5 * (double)wgs * k_in * (4.0 + 2.0 * m_rows);
     if (best == 0 || bytes / fill < best) best = bytes / fill, r = cand;
   }
+  if (m_rows > 8 && r == 4) r = 2;  // (four row blocks and sixteen batch rows do not fit the registers)
   const unsigned blocks = (unsigned)(groups * (4 / r));
-#define GQ_KNP_LAUNCH(R, XM)                                                                                  \
+#define GQ_KNP_LAUNCH(R, XM)                                                                                    \
   do {                                                                                                        \
     constexpr int lds_bytes = knp_lds_bytes(R, XM);                                                           \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                    \
@@ -299,10 +338,16 @@ int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const u
     else if (r == 2) GQ_KNP_LAUNCH(2, XM);         \
     else GQ_KNP_LAUNCH(1, XM);                     \
   } while (0)
+#define GQ_KNP_BY_R2(XM)                           \
+  do {                                             \
+    if (r == 2) GQ_KNP_LAUNCH(2, XM);              \
+    else GQ_KNP_LAUNCH(1, XM);                     \
+  } while (0)
   if (m_rows == 1) GQ_KNP_BY_R(1);
   else if (m_rows <= 4) GQ_KNP_BY_R(4);
   else if (m_rows <= 8) GQ_KNP_BY_R(8);
-  else GQ_KNP_BY_R(16);
+  else GQ_KNP_BY_R2(16);
+#undef GQ_KNP_BY_R2
 #undef GQ_KNP_BY_R
 #undef GQ_KNP_LAUNCH
   return check_launch("gemv_knp_kernel");
