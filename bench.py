@@ -347,6 +347,99 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                                        "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
                                        "roofline": hbm_roofline("gemv_mfma_kernel / gemv_stream_single_kernel (168 launches)", w_bytes, ms)}
+    # (1b) the same stack with every weight in the default layout of LinearGQ (groups along the output
+    # features), read from the derived copy a layer keeps after prepack_for_decode(): one launch of
+    # gq_linear_knp_act_f16 per matrix replayed from a HIP graph, and the same entries as a sequence
+    default_modes = ("default_layout_graph", "default_layout_sequence", "default_layout_two_entries_graph")
+    if modes is None or any(mode in modes for mode in default_modes):
+        # per layer: the six variables triples, packed [k_in, n_out / 64, 16]; roles q k v o up down
+        kn_vars, seed = [], 5000
+        for layer in range(n_layers):
+            for n_out, k_in in shapes:
+                seed += 1
+                kn_vars.append(pack_weight(make_weight(k_in, n_out, seed, False, device)))
+        torch.cuda.synchronize()
+
+        def graph_of(one_pass):
+            one_pass(stream_handle())
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                one_pass(stream_handle())
+            return graph
+
+        def knp(stream, x, w, y):
+            hip.call("gq_linear_knp_act_f16", x.data_ptr(), m_rows, w.blob.data_ptr(), 0, y.data_ptr(), w.n_out, w.k_in, GROUP, 0, stream)
+
+        if modes is None or "default_layout_graph" in modes or "default_layout_sequence" in modes:
+            blobs = [hip.prepack_gemv_kn(*v) for v in kn_vars]
+            if modes is None or "default_layout_graph" in modes:
+                def one_pass_default(stream):
+                    for i, w in enumerate(blobs):
+                        knp(stream, xs[w.k_in], w, ys[i % 6])
+
+                graph = graph_of(one_pass_default)
+                ms = time_launches(lambda _: graph.replay(), passes, warmup)
+                results["default_layout_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                                                   "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
+                                                   "roofline": hbm_roofline("gemv_knp_kernel (168 launches)", w_bytes, ms)}
+                del graph
+            if modes is None or "default_layout_sequence" in modes:
+                seq = hip.GemvSequence(device)
+                for i, w in enumerate(blobs):
+                    seq.add(xs[w.k_in], w, None, None, ys[i % 6], None, wait_previous=(i % 6) in (0, 3, 4, 5))
+                ms = time_launches(lambda _: seq.run(), passes, warmup)
+                torch.cuda.synchronize()
+                results["default_layout_sequence"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
+                                                      "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS, "status": int(seq.status.item()),
+                                                      "roofline": hbm_roofline("gemv_knp_kernel (sequence of 168 entries)", w_bytes, ms)}
+                del seq
+            del blobs
+            torch.cuda.empty_cache()
+        if modes is None or "default_layout_two_entries_graph" in modes:
+            # the decoder's data flow with two launches per layer: up | v | q | k stacked along the outputs
+            # (LinearGQ.fuse: the variables side by side along the group axis) reads the layer input, and the
+            # joint output product [down ; o] (LinearGQ.fuse_inputs: along the input features) reads
+            # up's and v's results, which lie end to end, and writes the next layer's input
+            first_w, out_w = [], []
+            for layer in range(n_layers):
+                q, k, v, o, up, down = (kn_vars[layer * 6 + role] for role in range(6))
+                first_w.append(hip.prepack_gemv_kn(*(torch.cat([up[part], v[part], q[part], k[part]], dim=1).contiguous() for part in range(3))))
+                # (scaled by 0.27 like the other layout's joint product: no normalisation layers here)
+                both = [torch.cat([down[part], o[part]], dim=0).contiguous() for part in range(3)]
+                out_w.append(hip.prepack_gemv_kn(both[0], (both[1].float() * 0.27).to(torch.float16), (both[2].float() * 0.27).to(torch.float16)))
+            torch.cuda.synchronize()
+            g.manual_seed(12)
+            h_in = (torch.randn((m_rows, hidden), generator=g, device=device, dtype=torch.float32) * 0.1).to(torch.float16)
+            wide = torch.empty((m_rows, ffn + 3 * hidden), dtype=torch.float16, device=device)
+            h_out = [torch.empty((m_rows, hidden), dtype=torch.float16, device=device) for _ in range(2)]
+            # (at one batch row x of the joint product is the first ffn + hidden values of the wide result;
+            # with more rows it is gathered by a copy, which stands for the attention and activation kernels
+            # that a model has between the two anyway)
+            joint_x = wide if m_rows == 1 else torch.empty((m_rows, ffn + hidden), dtype=torch.float16, device=device)
+
+            def one_pass_two(stream):
+                h = h_in
+                for layer in range(n_layers):
+                    knp(stream, h, first_w[layer], wide)
+                    if m_rows > 1:
+                        joint_x.copy_(wide[:, : ffn + hidden])
+                    h = h_out[layer % 2]
+                    hip.call("gq_linear_knp_act_f16", joint_x.data_ptr(), m_rows, out_w[layer].blob.data_ptr(), 0, h.data_ptr(), hidden,
+                             ffn + hidden, GROUP, 0, stream)
+
+            graph = graph_of(one_pass_two)
+            ms = time_launches(lambda _: graph.replay(), passes, warmup)
+            torch.cuda.synchronize()
+            finite = bool(torch.isfinite(h_out[(n_layers - 1) % 2].float()).all().item())
+            results["default_layout_two_entries_graph"] = {
+                "us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
+                "finite": finite, "roofline": hbm_roofline("gemv_knp_kernel (56 launches)", w_bytes, ms)}
+            if not finite:
+                raise SystemExit("bench.py: the default-layout stack produced values that are not finite")
+            del graph, first_w, out_w
+        del kn_vars
+        torch.cuda.empty_cache()
     # (2) the whole stack as one gq_gemv_sequence_f16 call, with the dependencies of a decoder layer
     # declared per entry.  Roles per layer, in `mats` order: q k v o up down.
     #   sequential block   q waits for the previous layer, k and v share its input, then o, up and
