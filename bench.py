@@ -706,10 +706,11 @@ def headline(result):
     if "gemv" in extra:  # configuration 3 (+ the stack's third shape): fraction of HBM peak on the packed weight
         short["c3_gemv"] = [_row(r, "hbm_frac") for r in extra["gemv"]]
     if "linear_knp" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out]), from the derived copy
-        short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_knp"]]
+        short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_knp"] if r["m"] <= 16]
+        short["c4_gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_knp"] if r["m"] > 16]
     if "linear_kn" in extra:  # ... and from the three variables as they are
         short["c3_gemv_default_layout_variables"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] <= 16]
-        short["gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
+        short["gemm_default_layout_variables"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
     if "gemm" in extra:  # configuration 4: fraction of the dense fp16 MFMA peak
         short["c4_gemm"] = [_row(r, "mfma_frac") for r in extra["gemm"]]
     if "stack" in extra:  # configuration 5: fraction of HBM peak on the packed weight
@@ -863,6 +864,13 @@ def main():
                 extra["linear_knp"].append(r)
                 log(f"  kn streaming layout gemv m={m} [{k_in}->{n_out}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
+        # prefill batches from the same copy (configuration 4 in the default layout): the MFMA pipeline of the other layout
+        for m in (128, 512, 2048):
+            r = bench_linear(hip, device, "gq_linear_knp_act_f16", m, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096),
+                             kernel="gemm_pipe2_kn_kernel")
+            extra["linear_knp"].append(r)
+            log(f"  kn streaming layout gemm m={m} [4096->16384]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
+            torch.cuda.empty_cache()
     if args.only in ("gemm", "all"):
         extra["gemm"] = []
         for m in (128, 512, 2048):

@@ -327,10 +327,13 @@ int gq_gemv_sequence_ws_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs
  *   gq_gemv_kn_prepack_f16      writes the blob (device memory, 16-byte aligned) from the variables
  *                               packed [k_in, n_out / 64, 16], scale / bias [k_in, n_out / 64] on `stream`
  *   gq_linear_knp_act_f16       y = act(x w + out_bias) as gq_linear_kn_act_f16 computes it, from the
- *                               blob, for 1 <= m_rows <= 16 (x, blob 16-byte aligned, y 8-byte); needs no
- *                               workspace and keeps no state.  The products x scale are rounded to
- *                               binary16 before they are multiplied with the exact codes; the result is
- *                               within the tolerance of the fused paths.
+ *                               blob, for any m_rows >= 1 (x, blob 16-byte aligned, y 8-byte); needs no
+ *                               workspace and keeps no state.  Up to 16 rows (and 17 to 32 as two passes)
+ *                               run the decode kernel: the products x scale are rounded to binary16
+ *                               before they are multiplied with the exact codes.  More rows run the
+ *                               pipelined MFMA kernel of gq_gemm_f16 with the blob as its weight source
+ *                               (every input feature brings its own scale and bias to the expansion).
+ *                               Either way the result is within the tolerance of the fused paths.
  */
 int64_t gq_gemv_kn_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size);
 int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob,

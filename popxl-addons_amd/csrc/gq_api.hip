@@ -385,10 +385,6 @@ int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, c
   if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: unknown activation %d", (int)activation);
   if (m_rows == 0 || n_out == 0) return GQ_OK;
-  if (m_rows > 16)
-    return gq::fail(GQ_ERR_UNSUPPORTED,
-                    "gq_linear_knp_act_f16: m_rows=%lld exceeds 16: the kn streaming layout serves decode batches; larger batches "
-                    "go through gq_linear_kn_act_f16 on the three variables", (long long)m_rows);
   if (!gq::gemv_kn_prepack_shape_ok(n_out, k_in, group_size))
     return gq::fail(GQ_ERR_UNSUPPORTED,
                     "gq_linear_knp_act_f16: the kn streaming layout needs group_size 64, n_out %% 64 == 0 and k_in %% 512 == 0 (got "
@@ -396,7 +392,17 @@ int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, c
   if (!x || !blob || !y) return gq::fail(GQ_ERR_NULL_POINTER, "gq_linear_knp_act_f16: x, blob and y must not be NULL");
   if (gq::misaligned(x, 16) || gq::misaligned(blob, 16) || gq::misaligned(y, 8) || gq::misaligned(out_bias, 2))
     return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_knp_act_f16: x and blob must be 16-byte aligned, y 8-byte, out_bias 2-byte");
-  return gq::launch_gemv_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
+  if (m_rows > (int64_t)1 << 30) return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: m_rows exceeds 2^30");
+  if (m_rows <= 16) return gq::launch_gemv_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
+  // 17 to 32 rows: two passes of the decode kernel over 16 rows each are faster than the prefill kernel's
+  // mostly empty tiles (as for the other layout)
+  if (m_rows <= 32) {
+    const int rc = gq::launch_gemv_knp(x, 16, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
+    if (rc != GQ_OK) return rc;
+    return gq::launch_gemv_knp(x + 16 * k_in, m_rows - 16, blob, out_bias, y + 16 * n_out, n_out, k_in, (int)activation,
+                               (hipStream_t)stream);
+  }
+  return gq::launch_gemm_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
 }
 
 int gq_compress_f16(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias,

@@ -90,6 +90,8 @@ int launch_gemv_kn_prepack(const uint16_t *packed, const uint16_t *scale, const 
                            int64_t k_in, hipStream_t stream);
 int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                     int64_t k_in, int act, hipStream_t stream);
+int launch_gemm_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                    int64_t k_in, int act, hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,
                     int64_t rows, int64_t n_groups, int64_t group_size, hipStream_t stream);
 int launch_compress_f32(const float *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,

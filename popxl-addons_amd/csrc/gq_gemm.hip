@@ -263,7 +263,41 @@ __device__ __forceinline__ half8_t dequant_result(const DequantState &st) {
                                  __builtin_shufflevector(st.w[2], st.w[3], 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-template <int WM, int WN, int FM, int FN, int XS, int KS>
+// The same for a word of the kn streaming layout (gq_gemv_kn.hip: weights grouped along the OUTPUT
+// features, the codes of an output contiguous along the input features).  Code e of a word sits in
+// nibble (3,7,2,6,1,5,0,4)[e], so the pair (2p, 2p+1) is the same nibble, 3 - p, of the two 16-bit
+// halves: a shift brings it to bits 3:0, one and-or puts both codes into the mantissas of 1024.0, one
+// packed add makes them exact, and one packed fma applies the pair's OWN scales and biases (every
+// input feature has its own in this layout): sq / zq hold (scale[k], scale[k+1]) for the four pairs.
+// (One mask and one magic number for all pairs: the 256 x 256 tile has no registers to spare.)
+struct KnMasks {
+  uint32_t mask, magic;  // in vector registers the compiler cannot see through (v_and_or_b32)
+};
+// LATE: the four fmas, which need the scales, are the last four operations (the scales are then
+// fetched while the first twelve run).
+template <int PIECES, bool LATE = false>
+__device__ __forceinline__ void dequant_piece_kn(int piece, uint32_t word, uint4_t sq, uint4_t zq, const KnMasks &km,
+                                                 DequantState &st) {
+  const half2_t kNeg1024 = {(half_t)-1024.0f, (half_t)-1024.0f};
+#pragma unroll
+  for (int op = 0; op < 16; ++op) {
+    if (op * PIECES / 16 != piece) continue;
+    const int p = LATE ? (op < 12 ? op / 3 : op - 12) : op >> 2, o = LATE ? (op < 12 ? op % 3 : 3) : op & 3;
+    if (o == 0) st.t[p] = p < 3 ? word >> (12 - 4 * p) : word;
+    if (o == 1) st.t[p] = (st.t[p] & km.mask) | km.magic;
+    if (o == 2) st.c[p] = as_half2(st.t[p]) + kNeg1024;
+    if (o == 3) st.w[p] = __builtin_elementwise_fma(st.c[p], as_half2(sq[p]), as_half2(zq[p]));
+  }
+}
+
+// KN: `packed` is the weight in the kn streaming layout (scale and bias are not read): lane (n, h) of a
+// fragment finds the 32 codes of output n at input features 64 T + 32 h .. of K tile T at
+//   unit (n / 64, T / 8) + 4096 ((n / 16) % 4) + 1024 ((T / 2) % 4) + 512 (T % 2) + 256 h + 16 (n % 16),
+// and the 64 scales (biases) of the tile at unit + 16384 (17408) + 128 (T % 8).  The 128 bytes of each
+// take the places in the wave's ring slot that the 32 scale (bias) dwords of the other layout take;
+// a lane reads the 16 bytes of its step's eight input features from them (all lanes of a half-wave
+// the same: a broadcast), one step ahead of the expansion that uses them.
+template <int WM, int WN, int FM, int FN, int XS, int KS, bool KN = false>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
@@ -300,13 +334,27 @@ __device__ __forceinline__ void gemm_pipe2_body(
 
   const uint4_t *b_src[FN];
   const uint32_t *s_src[FN], *z_src[FN];
+  const char *kn_codes[FN], *kn_scales[FN];  // KN: this lane's codes of K tile 0 / the fragment's scales of K tile 0
+  constexpr int kKnUnit = 18432;
 #pragma unroll
   for (int f = 0; f < FN; ++f) {
     const int row = min(n0 + wn * TN + f * 32 + fr, n_out - 1);
-    b_src[f] = packed + (int64_t)row * (k_in >> 5) + h + tile0 * 2;
-    s_src[f] = reinterpret_cast<const uint32_t *>(scale + (int64_t)row * groups_per_row);
-    z_src[f] = reinterpret_cast<const uint32_t *>(bias + (int64_t)row * groups_per_row);
+    if (KN) {
+      const int64_t chunks = k_in >> 9;
+      const int group = min((n0 + wn * TN + f * 32) >> 6, (n_out >> 6) - 1);  // (a fragment lies inside one group of 64)
+      kn_codes[f] = reinterpret_cast<const char *>(packed) + (int64_t)(row >> 6) * chunks * kKnUnit + ((row >> 4) & 3) * 4096 +
+                    h * 256 + (row & 15) * 16;
+      kn_scales[f] = reinterpret_cast<const char *>(packed) + (int64_t)group * chunks * kKnUnit + 16384 + (lane & 7) * 16;
+      b_src[f] = nullptr;
+      s_src[f] = z_src[f] = nullptr;
+    } else {
+      b_src[f] = packed + (int64_t)row * (k_in >> 5) + h + tile0 * 2;
+      s_src[f] = reinterpret_cast<const uint32_t *>(scale + (int64_t)row * groups_per_row);
+      z_src[f] = reinterpret_cast<const uint32_t *>(bias + (int64_t)row * groups_per_row);
+    }
   }
+  KnMasks km = {0x000F000Fu, 0x64006400u};
+  if (KN) asm volatile("" : "+v"(km.mask), "+v"(km.magic));
   char *w_ring = lds + KS * S::X_BYTES + (kgrp * NW + wave) * (kWStages * S::W_STAGE);
   const uint32_t w_rd = lds_base + KS * S::X_BYTES + (kgrp * NW + wave) * (kWStages * S::W_STAGE);
 
@@ -321,6 +369,24 @@ __device__ __forceinline__ void gemm_pipe2_body(
 #pragma unroll
     for (int q = 0; q < A_OPS; ++q)
       if (op == q) __builtin_amdgcn_global_load_lds(a_src[q] + t_load * 64, xs + (q * NW + wave) * 1024, 16, 0, 0);
+    if (KN) {
+      const int T = tile0 + t_load;  // K tile of the whole weight
+      const int64_t unit = (int64_t)(T >> 3) * kKnUnit;
+#pragma unroll
+      for (int f = 0; f < FN; ++f) {
+        if (op == A_OPS + f)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(kn_codes[f] + unit + ((T >> 1) & 3) * 1024 + (T & 1) * 512),
+                                           ws + f * 1024, 16, 0, 0);
+        // (eight lanes fetch the 128 bytes; like the 32 dword loads of the other layout, one instruction each)
+        if (op == A_OPS + FN + f && lane < 8)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(kn_scales[f] + unit + (T & 7) * 128),
+                                           ws + FN * 1024 + f * 128, 16, 0, 0);
+        if (op == A_OPS + 2 * FN + f && lane < 8)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(kn_scales[f] + unit + 1024 + (T & 7) * 128),
+                                           ws + FN * 1152 + f * 128, 16, 0, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int f = 0; f < FN; ++f) {
       if (op == A_OPS + f) __builtin_amdgcn_global_load_lds(b_src[f] + t_load * 2, ws + f * 1024, 16, 0, 0);
@@ -340,8 +406,19 @@ __device__ __forceinline__ void gemm_pipe2_body(
 #pragma unroll
     for (int f = 0; f < FN; ++f) {
       asm volatile("ds_read_b128 %0, %1" : "=v"(wq[f]) : "v"(ws + f * 1024 + lane * 16));
-      asm volatile("ds_read_b32 %0, %1" : "=v"(sw[f]) : "v"(ws + FN * 1024 + f * 128 + fr * 4));
-      asm volatile("ds_read_b32 %0, %1" : "=v"(zw[f]) : "v"(ws + FN * 1152 + f * 128 + fr * 4));
+      if (!KN) {
+        asm volatile("ds_read_b32 %0, %1" : "=v"(sw[f]) : "v"(ws + FN * 1024 + f * 128 + fr * 4));
+        asm volatile("ds_read_b32 %0, %1" : "=v"(zw[f]) : "v"(ws + FN * 1152 + f * 128 + fr * 4));
+      }
+    }
+  };
+  // KN: the scales and biases of the eight input features of MFMA step `step` of tile t (this lane's half h)
+  auto read_scales = [&](int t, int step, uint4_t (&sq)[FN], uint4_t (&zq)[FN]) {
+    const uint32_t ws = w_rd + (t % kWStages) * S::W_STAGE + h * 64 + step * 16;
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(sq[f]) : "v"(ws + FN * 1024 + f * 128));
+      asm volatile("ds_read_b128 %0, %1" : "=v"(zq[f]) : "v"(ws + FN * 1152 + f * 128));
     }
   };
   auto half_select = [&](int t) -> uint32_t {
@@ -363,14 +440,35 @@ __device__ __forceinline__ void gemm_pipe2_body(
   wait_vmcnt<OPS>();
   __builtin_amdgcn_s_barrier();
   uint4_t wq[FN], a[2][FM];
-  uint32_t sw[FN], zw[FN];
-  half2_t s2[FN], z2[FN];
+  uint32_t sw[FN] = {}, zw[FN] = {};
+  half2_t s2[FN] = {}, z2[FN] = {};
   half8_t b_cur[FN];
+  // KN: two sets of (scales, biases) of one MFMA step each: set [q] serves the steps of parity q of a
+  // tile (step 0 is expanded under step 3 of the tile before, step s + 1 under step s), and is
+  // fetched a step before it is used
+  // (Tiles with four or more A fragments per wave have no registers for two sets: ONE set, fetched
+  // at the start of the step whose expansion uses it, with the fmas that need it as the last of the
+  // sixteen operations and a counted wait in front of them.)
+  constexpr bool kOneSet = FM >= 4;
+  uint4_t sq[kOneSet ? 1 : 2][FN] = {}, zq[kOneSet ? 1 : 2][FN] = {};
   read_weights(0, wq, sw, zw);
+  if (KN) {
+    read_scales(0, 0, sq[0], zq[0]);
+    if (!kOneSet) read_scales(0, 1, sq[1], zq[1]);
+  }
 #pragma unroll
   for (int i = 0; i < FM; ++i)
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[0][i]) : "v"(a_rd_row + a_rd_chunk[0]), "n"(i * 4096));
-  {
+  if (KN) {
+#pragma unroll
+    for (int f = 0; f < FN; ++f) {
+      if (kOneSet) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(wq[f]), "+v"(sq[0][f]), "+v"(zq[0][f]) : "n"(FM));
+      else asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(wq[f]), "+v"(sq[0][f]), "+v"(zq[0][f]), "+v"(sq[kOneSet ? 0 : 1][f]), "+v"(zq[kOneSet ? 0 : 1][f]) : "n"(FM));
+      DequantState st0;
+      dequant_piece_kn<1>(0, wq[f][0], sq[0][f], zq[0][f], km, st0);
+      b_cur[f] = dequant_result(st0);
+    }
+  } else {
     const uint32_t sel = half_select(0);
 #pragma unroll
     for (int f = 0; f < FN; ++f) {
@@ -406,8 +504,24 @@ __device__ __forceinline__ void gemm_pipe2_body(
 #pragma unroll
         for (int o = 0; o < OPS_PER_GROUP; ++o)
           if ((s4 * FM + i) * OPS_PER_GROUP + o < OPS) issue_op((s4 * FM + i) * OPS_PER_GROUP + o, t_ahead, t + 2);
+        // KN: the scales of step s4 + 2 (of this tile: its ring slot is readable) go into the set that
+        // step s4's expansion, which is for step s4 + 1, does not use; they have landed by the next
+        // step's wait for this step's fragment reads
+        if (KN && i == 0) {
+          if (kOneSet) read_scales(t, s4 + 1, sq[0], zq[0]);  // (one set: of the step that is expanded now)
+          else if (s4 < 2) read_scales(t, s4 + 2, sq[s4 & 1], zq[s4 & 1]);
+        }
+        if (KN && kOneSet && i == FM - 2) {
+          // the fmas come in the last two groups: the set's reads are older than the FM - 2 fragment reads since
 #pragma unroll
-        for (int f = 0; f < FN; ++f) dequant_piece<FM>(i, wq[f][s4 + 1], s2[f], z2[f], st[f]);
+          for (int f = 0; f < FN; ++f) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(sq[0][f]), "+v"(zq[0][f]) : "n"(FM - 2));
+        }
+#pragma unroll
+        for (int f = 0; f < FN; ++f) {
+          if (KN && kOneSet) dequant_piece_kn<FM, true>(i, wq[f][s4 + 1], sq[0][f], zq[0][f], km, st[f]);
+          else if (KN) dequant_piece_kn<FM>(i, wq[f][s4 + 1], sq[(s4 + 1) & 1][f], zq[(s4 + 1) & 1][f], km, st[f]);
+          else dequant_piece<FM>(i, wq[f][s4 + 1], s2[f], z2[f], st[f]);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
       // keep this step's fragments allocated until here: a fragment read for the next step that
@@ -426,10 +540,14 @@ __device__ __forceinline__ void gemm_pipe2_body(
     __builtin_amdgcn_sched_barrier(0);
     uint4_t wq_next[FN];
     read_weights(t + 1, wq_next, sw, zw);
+    if (KN) {  // (the expansions that used the two sets are done: the last one ran under step 2)
+      read_scales(t + 1, 0, sq[0], zq[0]);
+      if (!kOneSet) read_scales(t + 1, 1, sq[1], zq[1]);
+    }
     const uint32_t xs_next = a_rd_row + ((t + 1) % XS) * S::X_STAGE;
-    const uint32_t sel_next = half_select(t + 1);
+    const uint32_t sel_next = KN ? 0u : half_select(t + 1);
     DequantState st[FN];
-    half2_t s2n[FN], z2n[FN];
+    half2_t s2n[FN] = {}, z2n[FN] = {};
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
       if (i + 1 < FM) asm volatile("" : "+v"(a[1][i]) : "v"(a[1][FM - 1]));
@@ -442,14 +560,22 @@ __device__ __forceinline__ void gemm_pipe2_body(
         // the weight reads are older than the two fragment reads issued since
 #pragma unroll
         for (int f = 0; f < FN; ++f) {
-          asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
-          s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
-          z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+          if (KN) {
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(wq_next[f]), "+v"(sq[0][f]), "+v"(zq[0][f]));
+            if (!kOneSet) asm volatile("" : "+v"(sq[kOneSet ? 0 : 1][f]), "+v"(zq[kOneSet ? 0 : 1][f]));
+          } else {
+            asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
+            s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
+            z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+          }
         }
       }
       if (i >= 2) {
 #pragma unroll
-        for (int f = 0; f < FN; ++f) dequant_piece<(FM > 2 ? FM - 2 : 1)>(i - 2, wq_next[f][0], s2n[f], z2n[f], st[f]);
+        for (int f = 0; f < FN; ++f) {
+          if (KN) dequant_piece_kn<(FM > 2 ? FM - 2 : 1)>(i - 2, wq_next[f][0], sq[0][f], zq[0][f], km, st[f]);
+          else dequant_piece<(FM > 2 ? FM - 2 : 1)>(i - 2, wq_next[f][0], s2n[f], z2n[f], st[f]);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -458,14 +584,22 @@ __device__ __forceinline__ void gemm_pipe2_body(
     if (FM == 1) {  // (the weight reads are older than the one fragment read issued since)
 #pragma unroll
       for (int f = 0; f < FN; ++f) {
-        asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
-        s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
-        z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+        if (KN) {
+          asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(wq_next[f]), "+v"(sq[0][f]), "+v"(zq[0][f]));
+          if (!kOneSet) asm volatile("" : "+v"(sq[kOneSet ? 0 : 1][f]), "+v"(zq[kOneSet ? 0 : 1][f]));
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(wq_next[f]), "+v"(sw[f]), "+v"(zw[f]));
+          s2n[f] = as_half2(__builtin_amdgcn_perm(sw[f], sw[f], sel_next));
+          z2n[f] = as_half2(__builtin_amdgcn_perm(zw[f], zw[f], sel_next));
+        }
       }
     }
     if (FM <= 2) {  // no MFMA group left to hide the expansion behind
 #pragma unroll
-      for (int f = 0; f < FN; ++f) dequant_piece<1>(0, wq_next[f][0], s2n[f], z2n[f], st[f]);
+      for (int f = 0; f < FN; ++f) {
+        if (KN) dequant_piece_kn<1>(0, wq_next[f][0], sq[0][f], zq[0][f], km, st[f]);
+        else dequant_piece<1>(0, wq_next[f][0], s2n[f], z2n[f], st[f]);
+      }
     }
 #pragma unroll
     for (int f = 0; f < FN; ++f) {
@@ -560,14 +694,20 @@ __device__ __forceinline__ void gemm_pipe2_body(
   }
 
   // D[m][n]: lane holds n = lane % 32 and m = 8 * (e / 4) + 4 * (lane / 32) + e % 4
+  // (The lane's position is worked out again from the thread index, through a register the compiler
+  // cannot see through: kept from the top of the kernel it would occupy registers across the K loop,
+  // which the largest tile does not have.)
+  int tid_e = tid;
+  asm volatile("" : "+v"(tid_e));
+  const int wave_e = (tid_e >> 6) % NW, wm_e = wave_e / WN, wn_e = wave_e % WN, fr_e = tid_e & 31, h_e = (tid_e >> 5) & 1;
   const bool interior = m0 + TILE_M <= m_rows && n0 + TILE_N <= n_out;
 #pragma unroll
   for (int f = 0; f < FN; ++f) {
-    const int n = n0 + wn * TN + f * 32 + fr;
+    const int n = n0 + wn_e * TN + f * 32 + fr_e;
     const float ob = (out_bias && n < n_out) ? (float)out_bias[n] : 0.f;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
-      half_t *dst = y + (int64_t)(m0 + wm * TM + i * 32 + 4 * h) * n_out + n;
+      half_t *dst = y + (int64_t)(m0 + wm_e * TM + i * 32 + 4 * h_e) * n_out + n;
       if (interior) {
 #pragma unroll
         for (int e = 0; e < 16; ++e)
@@ -575,7 +715,7 @@ __device__ __forceinline__ void gemm_pipe2_body(
       } else if (n < n_out) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int m = m0 + wm * TM + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+          const int m = m0 + wm_e * TM + i * 32 + 8 * (e >> 2) + 4 * h_e + (e & 3);
           if (m < m_rows) y[(int64_t)m * n_out + n] = (half_t)apply_activation(acc[i][f][e] + ob, act);
         }
       }
@@ -597,6 +737,15 @@ __global__ __launch_bounds__(KS * WM * WN * 64, OCC) void gemm_pipe2_kernel(cons
                                                                   unsigned *counters) {
   gemm_pipe2_body<WM, WN, FM, FN, XS, KS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, partial,
                                           counters);
+}
+
+// the same pipeline on a weight in the kn streaming layout (groups along the output features)
+template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS>
+__global__ __launch_bounds__(KS * WM * WN * 64, OCC) void gemm_pipe2_kn_kernel(const half_t *x, int m_rows, const uint4_t *blob,
+                                                                     const half_t *out_bias, half_t *y, int n_out, int k_in,
+                                                                     int act) {
+  gemm_pipe2_body<WM, WN, FM, FN, XS, KS, true>(x, m_rows, blob, nullptr, nullptr, out_bias, y, n_out, k_in, 6, act, nullptr,
+                                                nullptr);
 }
 
 namespace {
@@ -632,6 +781,30 @@ int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, cons
       reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act, partial,
       counters);
   return check_launch("gemm_pipe2_kernel");
+}
+
+template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS = 1>
+int launch_pipe2_kn(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                    int64_t k_in, int act, hipStream_t stream) {
+  using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
+  constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
+  auto kern = gemm_pipe2_kn_kernel<WM, WN, FM, FN, XS, OCC, KS>;
+  constexpr int kMaxDevices = 64;
+  static bool configured[kMaxDevices] = {false};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(GQ_ERR_NO_DEVICE, "no current device");
+  if (!configured[dev]) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute(lds=%d): %s", lds_bytes, hipGetErrorString(e));
+    configured[dev] = true;
+  }
+  const dim3 grid((unsigned)((n_out + TILE_N - 1) / TILE_N), (unsigned)((m_rows + TILE_M - 1) / TILE_M), 1u);
+  if (grid.y > 65535) return fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: m_rows=%lld too large", (long long)m_rows);
+  kern<<<grid, dim3(KS * WM * WN * 64), lds_bytes, stream>>>(
+      reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(blob),
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, act);
+  return check_launch("gemm_pipe2_kn_kernel");
 }
 
 }  // namespace
@@ -744,6 +917,21 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),
       reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act);
   return check_launch("gemm_tile_kernel");
+}
+
+// Prefill batches on a weight in the kn streaming layout (n_out % 64 == 0, k_in % 512 == 0, x and the blob
+// 16-byte aligned: the caller has checked): the pipelined kernel with the tile shape that plan_gemm
+// chooses for the other layout (K is not divided over workgroups: no workspace here).
+int launch_gemm_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                    int64_t k_in, int act, hipStream_t stream) {
+  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, false);
+#define GQ_PIPE2_KN(WM, WN, FM, FN, XS, OCC, ...) \
+  launch_pipe2_kn<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, blob, out_bias, y, n_out, k_in, act, stream)
+  if (plan.shape == 0) return GQ_PIPE2_KN(2, 2, 1, 1, 3, 2, 2);
+  if (plan.shape == 3) return GQ_PIPE2_KN(1, 8, 8, 1, 4, 2);
+  if (plan.shape == 2) return GQ_PIPE2_KN(1, 4, 8, 1, 3, 1);
+  return GQ_PIPE2_KN(2, 2, 2, 1, 3, 1, 2);
+#undef GQ_PIPE2_KN
 }
 
 }  // namespace gq

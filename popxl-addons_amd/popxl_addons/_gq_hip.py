@@ -223,8 +223,8 @@ def prepack_gemv_kn(packed, scale, bias):
 
 
 def linear_knp(x, weight, out_bias=None, activation=None, y=None):
-    """y = act(x @ w + out_bias) for x float16 [m_rows <= 16, k_in] on the GPU and a PrepackedWeight in
-    the kn streaming layout (gq_linear_knp_act_f16)."""
+    """y = act(x @ w + out_bias) for x float16 [m_rows, k_in] on the GPU and a PrepackedWeight in the kn
+    streaming layout (gq_linear_knp_act_f16: the decode kernel up to 16 rows, the MFMA pipeline above)."""
     import torch
 
     assert weight.layout == "kn" and x.is_cuda and x.is_contiguous() and x.shape[-1] == weight.k_in

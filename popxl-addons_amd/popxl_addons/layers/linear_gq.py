@@ -150,8 +150,8 @@ class LinearGQ:
                 ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None
                 _gq_hip.call("gq_linear_act_ws_f16", *args, 0 if ws is None else ws.data_ptr(),
                              0 if ws is None else ws.numel(), stream)
-            elif m_rows <= 16 and self._decode_copy is not None:
-                # groups along the output features, decode batch, the derived copy is there
+            elif self._decode_copy is not None:
+                # groups along the output features, the derived copy is there
                 _gq_hip.linear_knp(x2, self._decode_copy, b, act, y)
             else:
                 # groups along the output features: weight rows are input features
@@ -249,9 +249,9 @@ class LinearGQ:
 
     def prepack_for_decode(self):
         """dim=-1 / 1 (the default layout): keep a copy of the weight in the kn streaming layout, from
-        which `build` then serves batches of up to 16 rows (gq_linear_knp_act_f16: about twice as fast
-        as the kernel that reads the variables, at the price of a second copy of the packed weight);
-        larger batches still read the variables.  `load_weights` renews the copy.  Returns the copy
+        which `build` then serves every batch (gq_linear_knp_act_f16: decode batches about twice as
+        fast as the kernel that reads the variables, prefill batches through the MFMA pipeline of the
+        other layout; the price is a second copy of the packed weight).  `load_weights` renews the copy.  Returns the copy
         (a `_gq_hip.PrepackedWeight`, which `GemvSequence.add` accepts).  For dim=0 nothing is kept:
         the variables themselves are what the decode kernel reads."""
         if self.dim == 0:

@@ -42,7 +42,8 @@ def full_detail():
         "gemv": [_linear_row(m, n, k, "gemv_mfma_kernel / gemv_stream_single_kernel", "hbm") for n, k in shapes for m in (1, 8)],
         "linear_kn": [_linear_row(m, n, k, "gemv_kn_kernel", "hbm") for n, k in shapes for m in (1, 8)]
         + [_linear_row(128, 16384, 4096, "gemm_kn_tile_kernel", "mfma")],
-        "linear_knp": [_linear_row(m, n, k, "gemv_knp_kernel", "hbm") for n, k in shapes for m in (1, 8)],
+        "linear_knp": [_linear_row(m, n, k, "gemv_knp_kernel", "hbm") for n, k in shapes for m in (1, 8)]
+        + [_linear_row(m, 16384, 4096, "gemm_pipe2_kn_kernel", "mfma") for m in (128, 512, 2048)],
         "gemm": [_linear_row(m, 16384, 4096, "gemm_pipe2_kernel", "mfma") for m in (128, 512, 2048)],
         "gemm_other_shapes": [_linear_row(512, 4096, 4096, "gemm_pipe2_kernel", "mfma") for _ in range(7)],
         "stack": [_stack(m) for m in (1, 4, 8, 16)],
@@ -90,6 +91,7 @@ def test_headline_is_short_and_complete():
     assert len(back["extra"]["c3_gemv"]) == 6 and len(back["extra"]["c3_gemv_default_layout"]) == 6
     assert len(back["extra"]["c3_gemv_default_layout_variables"]) == 6
     assert [r["m"] for r in back["extra"]["c4_gemm"]] == [128, 512, 2048]
+    assert [r["m"] for r in back["extra"]["c4_gemm_default_layout"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c5_stack"]] == [1, 4, 8, 16]
     for r in back["extra"]["c5_stack"]:
         assert set(r) >= {"decoder", "no_waits", "per_launch_graph"}

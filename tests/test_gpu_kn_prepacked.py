@@ -85,6 +85,51 @@ def test_decode_shapes(hip, device, oracle, k_in, n_out, m_rows):
         assert_close(y.cpu().numpy(), oracle.np_linear(x, w_dec_t, ob), (k_in, n_out, m_rows, with_bias))
 
 
+@pytest.mark.parametrize("k_in,n_out", [(4096, 4096), (4096, 16384), (16384, 4096), (512, 64), (1536, 320), (1024, 4160)])
+@pytest.mark.parametrize("m_rows", [17, 31, 33, 64, 128, 200, 512])
+def test_prefill_shapes(hip, device, oracle, k_in, n_out, m_rows):
+    """More than 16 rows from the same copy: two passes of the decode kernel up to 32 rows, then the
+    pipelined MFMA kernel with every tile shape it has (64 x 64 ... 256 x 256, by batch and width),
+    ragged batches and widths that fill no whole tile."""
+    from popxl_addons._gq_hip import linear_knp
+
+    blob, _, w_dec_t = _weight(oracle, device, k_in, n_out, 11)
+    x = activations(m_rows, k_in, 14 + m_rows)
+    ob = np.random.default_rng(200 + m_rows).normal(0, 1, (n_out,)).astype(np.float16)
+    y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    linear_knp(to_dev(x, device), blob, to_dev(ob, device), None, y)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), oracle.np_linear(x, w_dec_t, ob), (k_in, n_out, m_rows))
+
+
+def test_benchmark_prefill_batches(hip, device, oracle):
+    """Benchmark configuration 4 in the default layout: 4096 -> 16384 at 1024 and 2048 rows (the 256 x 128 and
+    256 x 256 tiles), with an activation epilogue."""
+    from popxl_addons._gq_hip import linear_knp
+
+    k_in, n_out = 4096, 16384
+    blob, _, w_dec_t = _weight(oracle, device, k_in, n_out, 11)
+    for m_rows in (1024, 2048):
+        x = activations(m_rows, k_in, 15)
+        y = linear_knp(to_dev(x, device), blob, None, "relu")
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), oracle.np_linear(x, w_dec_t, None, "relu"), m_rows)
+
+
+@pytest.mark.parametrize("m_rows", [64, 300])
+def test_prefill_uneven_scales_and_biases(hip, device, oracle, m_rows):
+    """Scales and biases that vary by orders of magnitude between input features, through the MFMA
+    pipeline (every input feature applies its own to the codes)."""
+    from popxl_addons._gq_hip import linear_knp
+
+    k_in, n_out = 4096, 1024
+    blob, _, w_dec_t = _weight(oracle, device, k_in, n_out, 21, spread=True)
+    x = activations(m_rows, k_in, 23)
+    y = linear_knp(to_dev(x, device), blob)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), oracle.np_linear(x, w_dec_t, None), m_rows)
+
+
 @pytest.mark.parametrize("m_rows", [1, 8])
 def test_uneven_scales_and_biases(hip, device, oracle, m_rows):
     """Scales and biases that vary by orders of magnitude between input features: the activations are
@@ -142,9 +187,9 @@ def test_rejected_arguments(hip, device):
         assert lib.gq_gemv_kn_prepacked_bytes(n_out, k_in, gs) == GQ_ERR_UNSUPPORTED
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device=device)
     stream = torch.cuda.current_stream().cuda_stream
-    with pytest.raises(GQHipError) as e:  # more than 16 rows
-        hip.call("gq_linear_knp_act_f16", buf.data_ptr(), 17, buf.data_ptr(), 0, buf.data_ptr(), 64, 512, 64, 0, stream)
-    assert e.value.code == GQ_ERR_UNSUPPORTED and "gq_linear_kn_act_f16" in str(e.value)
+    with pytest.raises(GQHipError) as e:  # a group size the layout does not have
+        hip.call("gq_linear_knp_act_f16", buf.data_ptr(), 17, buf.data_ptr(), 0, buf.data_ptr(), 64, 512, 32, 0, stream)
+    assert e.value.code == GQ_ERR_UNSUPPORTED
     with pytest.raises(GQHipError) as e:
         hip.call("gq_linear_knp_act_f16", buf.data_ptr() + 2, 1, buf.data_ptr(), 0, buf.data_ptr(), 64, 512, 64, 0, stream)
     assert e.value.code == GQ_ERR_MISALIGNED
