@@ -454,7 +454,7 @@ __device__ __forceinline__ void gemm_pipe2_body(
   read_weights(0, wq, sw, zw);
   if (KN) {
     read_scales(0, 0, sq[0], zq[0]);
-    if (!kOneSet) read_scales(0, 1, sq[1], zq[1]);
+    if constexpr (!kOneSet) read_scales(0, 1, sq[1], zq[1]);
   }
 #pragma unroll
   for (int i = 0; i < FM; ++i)
@@ -542,7 +542,7 @@ __device__ __forceinline__ void gemm_pipe2_body(
     read_weights(t + 1, wq_next, sw, zw);
     if (KN) {  // (the expansions that used the two sets are done: the last one ran under step 2)
       read_scales(t + 1, 0, sq[0], zq[0]);
-      if (!kOneSet) read_scales(t + 1, 1, sq[1], zq[1]);
+      if constexpr (!kOneSet) read_scales(t + 1, 1, sq[1], zq[1]);
     }
     const uint32_t xs_next = a_rd_row + ((t + 1) % XS) * S::X_STAGE;
     const uint32_t sel_next = KN ? 0u : half_select(t + 1);

@@ -554,6 +554,75 @@ def test_gemv_sequence_random_graphs(hip, device, oracle, seed):
             assert_close(got, oracle.np_linear(x_dev.cpu().numpy(), w_dec, ob, act), (seed, i))
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_gemv_sequence_random_graphs_with_reused_buffers(hip, device, seed):
+    """Seeded random sequences in which outputs OVERWRITE buffers that earlier entries read or wrote
+    (what a model with one buffer per role does), declared as the interface asks: an entry waits for the
+    last entry that wrote its x and for the last entry that read or wrote the buffer it overwrites.
+    The host's plan of a launch has to tell exchanges from reported completion for every such case.
+    Checked against the same entries run one call at a time, in order, on a second set of buffers with
+    the same initial contents (the arithmetic of an entry is held to the oracle by the other tests;
+    this one holds the ORDER): every buffer ends with the values the in-order run leaves."""
+    from popxl_addons._gq_hip import GemvSequence, prepack_gemv
+
+    rng = np.random.default_rng(7000 + seed)
+    m_rows = int(rng.integers(1, 5))
+    widths = sorted({512 * int(rng.integers(1, 9)) for _ in range(3)})
+    n_entries = int(rng.integers(8, 20))
+    # two universes of buffers with the same contents: [0] the sequence's, [1] the in-order run's
+    buffers = []  # (width, [tensor, tensor])
+
+    def new_buffer(width, fill=None):
+        t = torch.full((m_rows, width), float("nan"), dtype=torch.float16, device=device) if fill is None else to_dev(fill, device)
+        buffers.append((width, [t, t.clone()]))
+        return len(buffers) - 1
+
+    for w in widths:
+        new_buffer(w, activations(m_rows, w, seed + w))
+    written = {i for i in range(len(buffers))}  # buffers that hold numbers
+    last_touch = {}  # buffer -> index of the last entry that read or wrote it
+    last_write = {}
+    seq = GemvSequence(device)
+    plan = []
+    for i in range(n_entries):
+        x_id = int(rng.choice(sorted(written)))
+        k_in = buffers[x_id][0]
+        n_out = int(rng.choice(widths))
+        candidates = [b for b, (w, _) in enumerate(buffers) if w == n_out and b != x_id and b >= len(widths)]
+        y_id = int(rng.choice(candidates)) if candidates and rng.random() < 0.5 else new_buffer(n_out)
+        w = rng.normal(0, 1.0 / np.sqrt(k_in), (n_out, k_in)).astype(np.float16)
+        pd, sd, bd = (to_dev(a, device) for a in group_quantize_compress_numpy(w, 64))
+        act = [None, "relu", "gelu_tanh"][int(rng.integers(0, 3))]
+        waits = [last_write.get(x_id), last_touch.get(y_id)]
+        waits = [v for v in waits if v is not None]
+        args = (prepack_gemv(pd, sd, bd), None, None) if rng.random() < 0.5 else (pd, sd, bd)
+        seq.add(buffers[x_id][1][0], *args, buffers[y_id][1][0], None, wait_for=max(waits) if waits else None, activation=act)
+        plan.append((x_id, y_id, (pd, sd, bd), n_out, k_in, act))
+        last_touch[x_id] = i
+        last_touch[y_id] = i
+        last_write[y_id] = i
+        written.add(y_id)
+    # the in-order run
+    stream = torch.cuda.current_stream().cuda_stream
+    for x_id, y_id, (pd, sd, bd), n_out, k_in, act in plan:
+        x, y = buffers[x_id][1][1], buffers[y_id][1][1]
+        hip.call("gq_linear_act_f16", x.data_ptr(), m_rows, pd.data_ptr(), sd.data_ptr(), bd.data_ptr(), 0, y.data_ptr(), n_out, k_in,
+                 64, hip.activation_code(act), stream)
+    torch.cuda.synchronize()
+    initial = [t[0].clone() for _, t in buffers]
+    for run in range(2):
+        for (_, t), first in zip(buffers, initial):
+            t[0].copy_(first)
+        seq.run()
+        seq.check()
+        for b, (_, (got, want)) in enumerate(buffers):
+            if b not in written:
+                continue
+            g, w_ = got.float().cpu().numpy(), want.float().cpu().numpy()
+            assert np.isfinite(g).all(), (seed, run, b)
+            assert np.abs(g - w_).max() <= 5e-3 * max(np.abs(w_).max(), 1e-3), (seed, run, b, np.abs(g - w_).max(), np.abs(w_).max())
+
+
 def test_gemv_sequence_fallback_and_graph(hip, device, oracle):
     """Shapes outside the persistent kernel (group 32) run entry by entry; the persistent kernel
     replays correctly from a captured graph."""
