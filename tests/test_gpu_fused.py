@@ -500,15 +500,30 @@ def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
         if not chained:
             for y2, ref in zip(outs2, refs):
                 assert_close(y2.cpu().numpy(), ref)
-    # a blob next to an entry that only the per-entry kernels can run (group 32) is refused
+    # a blob next to an entry that only the per-entry kernels can run (group 32): the sequence executes in
+    # runs -- the blob's entry on the persistent kernel, the other as a launch of its own
     rng = np.random.default_rng(4)
-    p32, s32, b32 = (to_dev(a, device) for a in group_quantize_compress_numpy(rng.normal(0, 0.02, (96, 256)).astype(np.float16), 32))
-    bad = GemvSequence(device)
+    w32 = rng.normal(0, 0.02, (96, 256)).astype(np.float16)
+    p32, s32, b32 = group_quantize_compress_numpy(w32, 32)
+    mixed_seq = GemvSequence(device)
     x, packed, scale, bias, y, ob = seq.keep[0]
-    bad.add(x, prepack_gemv(packed, scale, bias), None, None, y, ob)
-    bad.add(to_dev(activations(m_rows, 256, 1), device), p32, s32, b32, torch.empty((m_rows, 96), dtype=torch.float16, device=device))
+    want = y.clone()
+    y.fill_(float("nan"))
+    mixed_seq.add(x, prepack_gemv(packed, scale, bias), None, None, y, ob)
+    x32 = activations(m_rows, 256, 1)
+    y32 = torch.full((m_rows, 96), float("nan"), dtype=torch.float16, device=device)
+    mixed_seq.add(to_dev(x32, device), *(to_dev(a, device) for a in (p32, s32, b32)), y32)
+    mixed_seq.run()
+    mixed_seq.check()
+    top = want.float().abs().max().item()
+    assert (y.float() - want.float()).abs().max().item() <= 1.5e-3 * top
+    assert_close(y32.cpu().numpy(), oracle.np_linear(x32, oracle.np_decompress(p32, s32, b32)))
+    # what stays refused: a blob whose shape is outside the persistent kernel (more than four batch rows)
+    tall = GemvSequence(device)
+    x5 = to_dev(activations(5, x.shape[1], 2), device)
+    tall.add(x5, prepack_gemv(packed, scale, bias), None, None, torch.empty((5, packed.shape[0]), dtype=torch.float16, device=device))
     with pytest.raises(GQHipError) as e:
-        bad.run()
+        tall.run()
     assert "streaming layout" in str(e.value)
 
 

@@ -263,8 +263,15 @@ def test_prepacked_layer_in_a_sequence(hip, device):
     # the sequence kernel and the single-call kernels sum in different orders
     err = (y_down.float() - want.float()).abs().max().item() / want.float().abs().max().item()
     assert err <= 1e-2
-    with pytest.raises(NotImplementedError):
+    # a layer in the default layout has a streaming layout of its own (tests/test_gpu_kn_prepacked.py); what it cannot
+    # do is make one before it has variables, or for a group size the layout does not have
+    with pytest.raises(ValueError):
         LinearGQ(64, group_size=16, dim=-1).prepacked()
+    small = LinearGQ(64, group_size=16, dim=-1)
+    small.init_variables(512, torch.float16, device)
+    with pytest.raises(hip.GQHipError) as e:
+        small.prepacked()
+    assert e.value.code == hip.GQ_ERR_UNSUPPORTED
 
 
 def test_fuse_rejects_mismatched_layers(hip, device):
