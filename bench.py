@@ -337,7 +337,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
 
     results = {"m": m_rows, "entries": len(mats), "weight_bytes": w_bytes}
     # (1) one launch per matrix, replayed from a HIP graph
-    if modes is None:
+    if modes is None or "per_launch_graph" in modes:
         one_pass(stream_handle())
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -605,7 +605,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
                          "waits_per_pass": sum(1 for e in seq.entries if e[10] > 0),
                          # batch 1, every weight in the streaming layout, every dependency carried by data: the
                          # data-flow kernel; anything else: the LDS-ring kernel
-                         "roofline": hbm_roofline("gemv_flow_kernel" if m_rows == 1 and mode in FLOW_KERNEL_MODES else "gemv_stream_kernel",
+                         "roofline": hbm_roofline("gemv_mfma_kernel (one launch per entry)" if m_rows > 4 else
+                                                  "gemv_flow_kernel" if m_rows == 1 and mode in FLOW_KERNEL_MODES else "gemv_stream_kernel",
                                                   w_bytes, ms)}
         # the timed passes computed something: what the buffers hold now (the last layer's outputs)
         # equals single-call GEMVs on the same weights and the inputs the device had
@@ -686,7 +687,7 @@ def _stack_summary(r):
         out["decoder"] = {"us": round(us), "frac": round(r[mode]["hbm_frac"], 3), "kernel": r[mode]["roofline"]["kernel"],
                           "schedule": mode.replace("sequence_", "")}
     for key, mode in (("no_waits", "sequence_no_waits_streaming_layout"), ("per_launch_graph", "per_launch_graph"),
-                      ("default_layout", "default_layout_graph"), ("default_layout_sequence", "default_layout_sequence")):
+                      ("default_layout", "default_layout_graph"), ("default_layout_two_entries", "default_layout_two_entries_graph")):
         if mode in r:
             out[key] = {"us": round(r[mode]["us_per_pass"]), "frac": round(r[mode]["hbm_frac"], 3)}
     return out
@@ -754,7 +755,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--stack-modes", default="",
                     help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
-    ap.add_argument("--stack-batches", default="1,4", help="batch sizes of the stack runs")
+    ap.add_argument("--stack-batches", default="1,4,8", help="batch sizes of the stack runs")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
                     help="file for every figure of the run (the stdout line holds a summary); empty: no file")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -898,7 +899,11 @@ def main():
         for m in (int(v) for v in args.stack_batches.split(",")):
             # (a pass takes 0.5 to 1.6 ms; the first few dozen launches after a pause run up to 15 % slower
             # than the steady state, so they are warm-up)
-            r = bench_stack(hip, device, m, passes=100, warmup=40, modes=modes)
+            # (more than four batch rows: outside the persistent kernels, every entry is a launch of its own -- the
+            # graph of single launches, one sequence, and the default layout's graphs say what there is to say)
+            big = ("per_launch_graph", "sequence_parallel_block_fused_qkv_ffn_first", "default_layout_graph",
+                   "default_layout_two_entries_graph")
+            r = bench_stack(hip, device, m, passes=100, warmup=40, modes=modes if modes or m <= 4 else big)
             extra["stack"].append(r)
             for mode, v in r.items():
                 if isinstance(v, dict) and "us_per_pass" in v:
