@@ -256,11 +256,14 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     import torch
 
     knp = entry == "gq_linear_knp_act_f16"  # (the same layout, read from its derived copy: the kn streaming layout)
+    nkp = entry == "gq_linear_p_act_f16"  # (groups along k_in: the variables AND their derived copy in the streaming layout)
     kn = entry == "gq_linear_kn_act_f16" or knp
     sets = []
     for s in range(n_sets):
         w = make_weight(k_in, n_out, 200 + s, False, device) if kn else make_weight(n_out, k_in, 200 + s, False, device)
         sets.append((hip.prepack_gemv_kn(*pack_weight(w)),) if knp else pack_weight(w))
+        if nkp:
+            sets[-1] = sets[-1] + (hip.prepack_gemv(*sets[-1]),)
     g = torch.Generator(device=device)
     g.manual_seed(7)
     x = torch.randn((m_rows, k_in), generator=g, device=device, dtype=torch.float32).to(torch.float16)
@@ -274,6 +277,11 @@ def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets,
     def step(i):
         if knp:
             hip.call(entry, x.data_ptr(), m_rows, sets[i % n_sets][0].blob.data_ptr(), 0, y.data_ptr(), n_out, k_in, GROUP, 0, stream)
+            return
+        if nkp:
+            p, s, b, copy = sets[i % n_sets]
+            hip.call(entry, x.data_ptr(), m_rows, p.data_ptr(), s.data_ptr(), b.data_ptr(), copy.blob.data_ptr(), 0, y.data_ptr(), n_out,
+                     k_in, GROUP, 0, 0, 0, stream)
             return
         p, s, b = sets[i % n_sets]
         if kn:
@@ -709,11 +717,13 @@ def headline(result):
     if "linear_knp" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out]), from the derived copy
         short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_knp"] if r["m"] <= 16]
         short["c4_gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_knp"] if r["m"] > 16]
-    if "linear_kn" in extra:  # ... and from the three variables as they are
-        short["c3_gemv_default_layout_variables"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] <= 16]
+    if "linear_kn" in extra:  # ... and from the three variables as they are (the other batches: in the detail file)
+        short["c3_gemv_default_layout_variables"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] == 1]
         short["gemm_default_layout_variables"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
     if "gemm" in extra:  # configuration 4: fraction of the dense fp16 MFMA peak
         short["c4_gemm"] = [_row(r, "mfma_frac") for r in extra["gemm"]]
+    if "gemm_streaming_layout" in extra:  # ... the same with the weight's derived copy beside the variables
+        short["c4_gemm_streaming_layout"] = [_row(r, "mfma_frac") for r in extra["gemm_streaming_layout"]]
     if "stack" in extra:  # configuration 5: fraction of HBM peak on the packed weight
         short["c5_stack"] = [_stack_summary(r) for r in extra["stack"]]
     out = {k: v for k, v in result.items() if k not in ("extra", "cpu_baseline", "roofline")}
@@ -879,6 +889,15 @@ def main():
             r = bench_linear(hip, device, "gq_gemm_f16", m, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096), kernel="gemm_pipe2_kernel")
             extra["gemm"].append(r)
             log(f"  gemm m={m} [16384x4096]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
+            torch.cuda.empty_cache()
+        # the same three batches when the caller also holds the weight in the streaming layout (what LinearGQ(dim=0) does
+        # after prepack_for_decode()): the same kernel and the same bits, the weight pieces 512 bytes contiguous
+        extra["gemm_streaming_layout"] = []
+        for m in (128, 512, 2048):
+            r = bench_linear(hip, device, "gq_linear_p_act_f16", m, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096),
+                             kernel="gemm_pipe2_kernel (streaming layout)")
+            extra["gemm_streaming_layout"].append(r)
+            log(f"  gemm, streaming layout m={m} [16384x4096]: {r['us']:.1f} us, {r['tflops']:.0f} TFLOP/s ({r['mfma_frac']:.1%} of fp16 dense peak)")
             torch.cuda.empty_cache()
         # the stack's other layer shapes (4096 outputs: few tiles, where the choice of tile matters most) and the
         # batches between the GEMV's 16 rows and full GEMM tiles, through the entry that the layer calls

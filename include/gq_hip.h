@@ -151,6 +151,22 @@ int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                          int64_t workspace_bytes, void *stream);
 
 /*
+ * gq_linear_act_ws_f16 for a caller that also holds the weight's derived copy in the streaming layout
+ * (`blob`, made by gq_gemv_prepack_f16 below from the same packed, scale and bias: group_size 64,
+ * k_in % 512 == 0, 16-byte aligned).  No counterpart in the reference (LinearGQ.build reads the three
+ * variables, popxl_addons/layers/linear_gq.py:99-109).  Batches of more than 16 rows that run the
+ * pipelined GEMM kernel then read the copy, whose pieces are 512 bytes contiguous where a row of
+ * `packed` contributes 32 bytes per step of 64 input features: the same results to the tolerance of
+ * the fused paths, 5 - 12 % sooner.  Every other path (m_rows <= 16, passes of the GEMV kernel, shapes
+ * outside the pipelined kernel) reads packed, scale and bias as gq_linear_act_ws_f16 does, so these
+ * stay required.  blob == NULL: the call is gq_linear_act_ws_f16.
+ */
+int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                        const uint16_t *bias, const void *blob, const uint16_t *out_bias, uint16_t *y,
+                        int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation, void *workspace,
+                        int64_t workspace_bytes, void *stream);
+
+/*
  * Fused decompress + matmul, groups along the OUTPUT features: the computation of LinearGQ.build
  * with dim = -1 or 1, the constructor default (popxl_addons/layers/linear_gq.py:26, 59-62, 99-109):
  *   w = decompress(packed, scale, bias)      [k_in, n_out]

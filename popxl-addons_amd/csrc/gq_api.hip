@@ -162,11 +162,24 @@ int64_t gq_gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int
 int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                          const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                          int64_t group_size, int32_t activation, void *workspace, int64_t workspace_bytes, void *stream) {
+  return gq_linear_p_act_f16(x, m_rows, packed, scale, bias, nullptr, out_bias, y, n_out, k_in, group_size, activation, workspace,
+                             workspace_bytes, stream);
+}
+
+int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
+                        const uint16_t *bias, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
+                        int64_t k_in, int64_t group_size, int32_t activation, void *workspace, int64_t workspace_bytes,
+                        void *stream) {
   const int rc = gq::check_linear_args("gq_linear_act_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
                                        k_in, group_size);
   if (rc <= 0) return rc;
   if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_act_f16: unknown activation %d", (int)activation);
+  if (blob) {
+    const int64_t blob_bytes = gq_gemv_prepacked_bytes(n_out, k_in, group_size);
+    if (blob_bytes < 0) return (int)blob_bytes;  // (no streaming layout for this shape: the message is set)
+    if (gq::misaligned(blob, 16)) return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_p_act_f16: blob must be 16-byte aligned");
+  }
   // the workspace is an option: one that is missing, misaligned or too small is not used
   if (m_rows <= 16 || !workspace || gq::misaligned(workspace, 16) ||
       workspace_bytes < gq_gemm_workspace_bytes(m_rows, n_out, k_in, group_size))
@@ -179,7 +192,7 @@ int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
                              workspace != nullptr, (hipStream_t)stream, &passes_rc))
     return passes_rc;
   return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation, workspace,
-                         (hipStream_t)stream);
+                         (hipStream_t)stream, blob);
 }
 
 int64_t gq_linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {

@@ -51,9 +51,10 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream);
 // workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
+// blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16, which the pipelined kernel then reads
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, void *workspace, hipStream_t stream);
+                int64_t group_size, int act, void *workspace, hipStream_t stream, const void *blob = nullptr);
 int64_t gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size);
 double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split);
 // Batches of 17 to 128 rows as passes of the GEMV kernel over 16 rows each, where that is expected

@@ -297,7 +297,7 @@ __device__ __forceinline__ void dequant_piece_kn(int piece, uint32_t word, uint4
 // take the places in the wave's ring slot that the 32 scale (bias) dwords of the other layout take;
 // a lane reads the 16 bytes of its step's eight input features from them (all lanes of a half-wave
 // the same: a broadcast), one step ahead of the expansion that uses them.
-template <int WM, int WN, int FM, int FN, int XS, int KS, bool KN = false>
+template <int WM, int WN, int FM, int FN, int XS, int KS, bool KN = false, bool BLOB = false>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
@@ -335,7 +335,7 @@ __device__ __forceinline__ void gemm_pipe2_body(
   const uint4_t *b_src[FN];
   const uint32_t *s_src[FN], *z_src[FN];
   const char *kn_codes[FN], *kn_scales[FN];  // KN: this lane's codes of K tile 0 / the fragment's scales of K tile 0
-  constexpr int kKnUnit = 18432;
+  constexpr int kKnUnit = 18432, kStreamItem = 4608;
 #pragma unroll
   for (int f = 0; f < FN; ++f) {
     const int row = min(n0 + wn * TN + f * 32 + fr, n_out - 1);
@@ -347,7 +347,16 @@ __device__ __forceinline__ void gemm_pipe2_body(
       kn_scales[f] = reinterpret_cast<const char *>(packed) + (int64_t)group * chunks * kKnUnit + 16384 + (lane & 7) * 16;
       b_src[f] = nullptr;
       s_src[f] = z_src[f] = nullptr;
+    } else if (BLOB) {
+      // the items of the row's block of 16 (4608 bytes per 512 input features): this lane's 16 bytes of K tile 0,
+      // and the row's 16 bytes of scales (8 groups; the biases 256 bytes on) of the first item
+      const char *const items = reinterpret_cast<const char *>(packed) + (int64_t)(row >> 4) * (k_in >> 9) * kStreamItem;
+      kn_codes[f] = items + h * 256 + (row & 15) * 16;
+      kn_scales[f] = items + 4096 + (row & 15) * 16;
+      b_src[f] = nullptr;
+      s_src[f] = z_src[f] = nullptr;
     } else {
+      kn_codes[f] = kn_scales[f] = nullptr;
       b_src[f] = packed + (int64_t)row * (k_in >> 5) + h + tile0 * 2;
       s_src[f] = reinterpret_cast<const uint32_t *>(scale + (int64_t)row * groups_per_row);
       z_src[f] = reinterpret_cast<const uint32_t *>(bias + (int64_t)row * groups_per_row);
@@ -384,6 +393,23 @@ __device__ __forceinline__ void gemm_pipe2_body(
         if (op == A_OPS + 2 * FN + f && lane < 8)
           __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(kn_scales[f] + unit + 1024 + (T & 7) * 128),
                                            ws + FN * 1152 + f * 128, 16, 0, 0);
+      }
+      return;
+    }
+    if (BLOB) {
+      const int T = tile0 + t_load;  // K tile of the whole weight; its group of 64 is number T % 8 of the item
+      const int64_t item = (int64_t)(T >> 3) * kStreamItem;
+#pragma unroll
+      for (int f = 0; f < FN; ++f) {
+        if (op == A_OPS + f)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4_t *>(kn_codes[f] + item + ((T >> 1) & 3) * 1024 + (T & 1) * 512),
+                                           ws + f * 1024, 16, 0, 0);
+        if (op == A_OPS + FN + f && h == 0)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(kn_scales[f] + item + ((T & 7) >> 1) * 4),
+                                           ws + FN * 1024 + f * 128, 4, 0, 0);
+        if (op == A_OPS + 2 * FN + f && h == 0)
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(kn_scales[f] + item + 256 + ((T & 7) >> 1) * 4),
+                                           ws + FN * 1152 + f * 128, 4, 0, 0);
       }
       return;
     }
@@ -729,14 +755,15 @@ __device__ __forceinline__ void gemm_pipe2_body(
 
 // (external linkage: their address is taken on the host for hipFuncSetAttribute)
 // OCC: waves per SIMD the register budget is sized for (2: 256 registers per lane, 1: 512)
-template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS>
+// BLOB: `packed` is the weight in the streaming layout of gq_gemv_prepack_f16 (scale and bias are not read)
+template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS, bool BLOB>
 __global__ __launch_bounds__(KS * WM * WN * 64, OCC) void gemm_pipe2_kernel(const half_t *x, int m_rows, const uint4_t *packed,
                                                                   const half_t *scale, const half_t *bias,
                                                                   const half_t *out_bias, half_t *y, int n_out,
                                                                   int k_in, int gs_shift, int act, float4_t *partial,
                                                                   unsigned *counters) {
-  gemm_pipe2_body<WM, WN, FM, FN, XS, KS>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, partial,
-                                          counters);
+  gemm_pipe2_body<WM, WN, FM, FN, XS, KS, false, BLOB>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act,
+                                                       partial, counters);
 }
 
 // the same pipeline on a weight in the kn streaming layout (groups along the output features)
@@ -752,14 +779,14 @@ namespace {
 
 constexpr int kGemmCounters = 4096;  // arrival counters at the start of a workspace (16 KiB), one per output tile
 
-template <int WM, int WN, int FM, int FN, int XS, int OCC, int KS = 1>
+template <bool BLOB, int WM, int WN, int FM, int FN, int XS, int OCC, int KS = 1>
 int launch_pipe2(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                  const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int gs_shift,
                  int act, int z_splits, void *workspace, hipStream_t stream) {
   using S = Pipe2Shape<WM, WN, FM, FN, XS, KS>;
   constexpr int TILE_M = S::TILE_M, TILE_N = S::TILE_N, lds_bytes = S::LDS_BYTES;
   static_assert(lds_bytes <= 160 * 1024, "LDS budget of a gfx950 compute unit");
-  auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC, KS>;
+  auto kern = gemm_pipe2_kernel<WM, WN, FM, FN, XS, OCC, KS, BLOB>;
   // the attribute belongs to the (function, device) pair; same value every time: a benign race
   constexpr int kMaxDevices = 64;
   static bool configured[kMaxDevices] = {false};
@@ -887,18 +914,24 @@ int64_t gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_
 
 // `workspace`: NULL, or gemm_workspace_bytes() bytes of device memory whose first 16 KiB (the counters)
 // are zero; the kernel leaves them zero.
+// `blob`: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16 (group_size 64, k_in % 512 == 0,
+// 16-byte aligned: the caller has checked); the pipelined kernel then reads it instead of the three variables.
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, void *workspace, hipStream_t stream) {
+                int64_t group_size, int act, void *workspace, hipStream_t stream, const void *blob) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % BK == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
   if (!fast_ok)
     return launch_gemv_generic_rows(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
   const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
-#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...)                                                                            \
-  launch_pipe2<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, gs_shift, act, \
-                                                       plan.splits, plan.splits > 1 ? workspace : nullptr, stream)
+#define GQ_PIPE2(WM, WN, FM, FN, XS, OCC, ...)                                                                              \
+  (blob ? launch_pipe2<true, WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, static_cast<const uint16_t *>(blob), nullptr,    \
+                                                                     nullptr, out_bias, y, n_out, k_in, gs_shift, act,           \
+                                                                     plan.splits, plan.splits > 1 ? workspace : nullptr, stream) \
+        : launch_pipe2<false, WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in,  \
+                                                                      gs_shift, act, plan.splits,                                \
+                                                                      plan.splits > 1 ? workspace : nullptr, stream))
   if (gemm_pipelined_ok(x, packed, scale, bias, k_in, group_size)) {
     const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, workspace != nullptr);
     if (plan.shape == 0) return GQ_PIPE2(2, 2, 1, 1, 3, 2, 2);  // 64 x 64, two groups of 4 waves of 32 x 32

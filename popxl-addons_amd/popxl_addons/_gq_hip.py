@@ -42,6 +42,7 @@ EXPORTS = (
     "gq_linear_act_f16",
     "gq_gemm_workspace_bytes",
     "gq_linear_act_ws_f16",
+    "gq_linear_p_act_f16",
     "gq_linear_kn_workspace_bytes",
     "gq_linear_kn_act_f16",
     "gq_linear_kn_act_noalloc_f16",
@@ -105,6 +106,8 @@ def load():
     lib.gq_gemm_workspace_bytes.restype = i64
     lib.gq_linear_act_ws_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
     lib.gq_linear_act_ws_f16.restype = ctypes.c_int
+    lib.gq_linear_p_act_f16.argtypes = [p, i64, p, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
+    lib.gq_linear_p_act_f16.restype = ctypes.c_int
     lib.gq_linear_kn_workspace_bytes.argtypes = [i64, i64, i64, i64]
     lib.gq_linear_kn_workspace_bytes.restype = i64
     lib.gq_linear_kn_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
@@ -176,7 +179,8 @@ def linear_kn_workspace(device, nbytes):
 class PrepackedWeight:
     """One weight in a streaming layout: a device blob derived from the three LinearGQ variables.
     layout "nk": groups along the input features (LinearGQ dim=0), made by prepack_gemv(), read by
-    GemvSequence entries only; layout "kn": groups along the output features (dim=-1 / 1, the
+    GemvSequence entries and, beside the variables, by gq_linear_p_act_f16's GEMM kernel; layout "kn":
+    groups along the output features (dim=-1 / 1, the
     default), made by prepack_gemv_kn(), read by GemvSequence entries and by linear_knp()."""
 
     def __init__(self, blob, n_out, k_in, group_size, layout="nk"):

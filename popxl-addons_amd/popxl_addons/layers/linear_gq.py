@@ -55,7 +55,7 @@ class LinearGQ:
         self.group_size = group_size
         self.dim = dim
         self.variables: Optional[NamedTensors] = None
-        self._decode_copy = None  # dim=-1 / 1 only: the weight in the kn streaming layout (prepack_for_decode)
+        self._decode_copy = None  # the weight in the streaming layout of its dim, once prepack_for_decode has made it
 
     # ----------------------------------------------------------------------------- variables
 
@@ -148,7 +148,9 @@ class LinearGQ:
                 # (few output tiles: several workgroups divide the input features of a tile through a workspace)
                 need = _gq_hip.load().gq_gemm_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)
                 ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None
-                _gq_hip.call("gq_linear_act_ws_f16", *args, 0 if ws is None else ws.data_ptr(),
+                # (with the derived copy the pipelined GEMM kernel reads that; everything else reads the variables)
+                blob = 0 if self._decode_copy is None else self._decode_copy.blob.data_ptr()
+                _gq_hip.call("gq_linear_p_act_f16", *args[:5], blob, *args[5:], 0 if ws is None else ws.data_ptr(),
                              0 if ws is None else ws.numel(), stream)
             elif self._decode_copy is not None:
                 # groups along the output features, the derived copy is there
@@ -248,14 +250,16 @@ class LinearGQ:
         return make(v.weight_compressed.data, v.weight_decompression_scale.data, v.weight_decompression_bias.data)
 
     def prepack_for_decode(self):
-        """dim=-1 / 1 (the default layout): keep a copy of the weight in the kn streaming layout, from
-        which `build` then serves every batch (gq_linear_knp_act_f16: decode batches about twice as
-        fast as the kernel that reads the variables, prefill batches through the MFMA pipeline of the
-        other layout; the price is a second copy of the packed weight).  `load_weights` renews the copy.  Returns the copy
-        (a `_gq_hip.PrepackedWeight`, which `GemvSequence.add` accepts).  For dim=0 nothing is kept:
-        the variables themselves are what the decode kernel reads."""
-        if self.dim == 0:
-            return self.prepacked()
+        """Keep a copy of the weight in the streaming layout of its dim (the price: a second copy of
+        the packed weight); `load_weights` renews it.  Returns the copy (a `_gq_hip.PrepackedWeight`,
+        which `GemvSequence.add` accepts).
+
+        dim=-1 / 1 (the default layout): `build` then serves every batch from the copy
+        (gq_linear_knp_act_f16: decode batches about twice as fast as the kernel that reads the
+        variables, prefill batches through the MFMA pipeline of the other layout).
+        dim=0: `build` hands the copy to gq_linear_p_act_f16 beside the variables; batches that run the
+        pipelined GEMM kernel read it (5 - 12 % sooner, the same bits), single decode calls read the
+        variables as before, and a `GemvSequence` streams the copy."""
         self._decode_copy = self.prepacked()
         return self._decode_copy
 

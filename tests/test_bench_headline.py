@@ -45,6 +45,7 @@ def full_detail():
         "linear_knp": [_linear_row(m, n, k, "gemv_knp_kernel", "hbm") for n, k in shapes for m in (1, 8)]
         + [_linear_row(m, 16384, 4096, "gemm_pipe2_kn_kernel", "mfma") for m in (128, 512, 2048)],
         "gemm": [_linear_row(m, 16384, 4096, "gemm_pipe2_kernel", "mfma") for m in (128, 512, 2048)],
+        "gemm_streaming_layout": [_linear_row(m, 16384, 4096, "gemm_pipe2_kernel (streaming layout)", "mfma") for m in (128, 512, 2048)],
         "gemm_other_shapes": [_linear_row(512, 4096, 4096, "gemm_pipe2_kernel", "mfma") for _ in range(7)],
         "stack": [_stack(m) for m in (1, 4, 8, 16)],
         "bench_wall_s": 123.4,
@@ -89,9 +90,10 @@ def test_headline_is_short_and_complete():
     assert "legs" not in back["cpu_baseline"]
     # one short record per benchmark shape of configurations 3, 4 and 5
     assert len(back["extra"]["c3_gemv"]) == 6 and len(back["extra"]["c3_gemv_default_layout"]) == 6
-    assert len(back["extra"]["c3_gemv_default_layout_variables"]) == 6
+    assert len(back["extra"]["c3_gemv_default_layout_variables"]) == 3  # (batch 1 only: the rest is in the detail file)
     assert [r["m"] for r in back["extra"]["c4_gemm"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c4_gemm_default_layout"]] == [128, 512, 2048]
+    assert [r["m"] for r in back["extra"]["c4_gemm_streaming_layout"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c5_stack"]] == [1, 4, 8, 16]
     for r in back["extra"]["c5_stack"]:
         assert set(r) >= {"decoder", "no_waits", "per_launch_graph"}

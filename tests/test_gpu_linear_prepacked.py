@@ -1,0 +1,122 @@
+"""gq_linear_p_act_f16: the fused matmul for weights grouped along the input features (LinearGQ with
+dim=0) when the caller also holds the derived copy in the streaming layout (gq_gemv_prepack_f16).
+The pipelined GEMM kernel then reads the copy; the arithmetic is that of gq_linear_act_ws_f16 on the
+three variables, so the results are the oracle's to the tolerance of the fused paths AND equal to
+that entry point's bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from gq_testlib import activations, assert_bits_equal, normal_weight, to_dev
+from popxl_addons._gq_hip import GQ_ERR_MISALIGNED, GQ_ERR_UNSUPPORTED, GQHipError
+from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy
+from test_gpu_fused import assert_close
+
+pytestmark = pytest.mark.gpu
+
+_WEIGHTS = {}
+
+
+def _weight(hip, device, oracle, n_out, k_in, seed):
+    key = (n_out, k_in, seed)
+    if key not in _WEIGHTS:
+        packed, scale, bias = group_quantize_compress_numpy(normal_weight(n_out, k_in, seed), 64)
+        dev = tuple(to_dev(a, device) for a in (packed, scale, bias))
+        _WEIGHTS[key] = (dev, hip.prepack_gemv(*dev), oracle.np_decompress(packed, scale, bias))
+    return _WEIGHTS[key]
+
+
+def _run(hip, device, x, dev, blob, out_bias, n_out, k_in, act, workspace=None):
+    xd = to_dev(x, device)
+    od = None if out_bias is None else to_dev(out_bias, device)
+    y = torch.full((x.shape[0], n_out), float("nan"), dtype=torch.float16, device=device)
+    hip.call("gq_linear_p_act_f16", xd.data_ptr(), x.shape[0], dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(),
+             0 if blob is None else blob.data_ptr(), 0 if od is None else od.data_ptr(), y.data_ptr(), n_out, k_in, 64, act,
+             0 if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel(),
+             torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("m_rows", [128, 512, 2048])
+def test_benchmark_prefill_batches(hip, device, oracle, m_rows):
+    """Benchmark configuration 4 on the derived copy: every tile shape of the pipelined kernel."""
+    n_out, k_in = 16384, 4096
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 21)
+    x = activations(m_rows, k_in, 22)
+    ob = np.random.default_rng(23).normal(0, 1, (n_out,)).astype(np.float16) if m_rows == 512 else None
+    y = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 0)
+    assert_close(y, oracle.np_linear(x, w_dec, ob), m_rows)
+    assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 0), "against the variables")
+
+
+@pytest.mark.parametrize("n_out,k_in,m_rows", [(4096, 4096, 300), (4096, 16384, 128), (4104, 512, 300), (8200, 1024, 777),
+                                               (4104, 1536, 2060), (1000, 4096, 40), (72, 512, 33), (16384, 4096, 64),
+                                               (4096, 4096, 17), (4096, 4096, 8)])
+def test_shapes_with_and_without_workspace(hip, device, oracle, n_out, k_in, m_rows):
+    """Ragged tiles and row blocks (n_out not a multiple of 16: the copy pads the last block), K divided
+    over workgroups through the workspace, the 64 x 64 tiles, batches that run as passes of the GEMV
+    kernel or as one GEMV (those read the variables whether the copy is there or not), an activation."""
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 31)
+    x = activations(m_rows, k_in, 32)
+    ob = np.random.default_rng(33).normal(0, 1, (n_out,)).astype(np.float16)
+    need = hip.load().gq_gemm_workspace_bytes(m_rows, n_out, k_in, 64)
+    ws = torch.zeros(max(need, 16384), dtype=torch.uint8, device=device)
+    y_ref = oracle.np_linear(x, w_dec, ob, "gelu_tanh")
+    for workspace in (None, ws):
+        y = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 2, workspace)
+        assert_close(y, y_ref, (n_out, k_in, m_rows, workspace is not None))
+        assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 2, workspace), "against the variables")
+        assert not ws[:16384].any(), "arrival counters must be back at zero"
+
+
+def test_without_the_copy_it_is_the_workspace_entry_point(hip, device, oracle):
+    n_out, k_in, m_rows = 4096, 4096, 256
+    dev, _, _ = _weight(hip, device, oracle, n_out, k_in, 31)
+    x = activations(m_rows, k_in, 34)
+    xd = to_dev(x, device)
+    y = torch.empty((m_rows, n_out), dtype=torch.float16, device=device)
+    hip.call("gq_linear_act_ws_f16", xd.data_ptr(), m_rows, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(), 0,
+             y.data_ptr(), n_out, k_in, 64, 1, 0, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert_bits_equal(_run(hip, device, x, dev, None, None, n_out, k_in, 1), y.cpu().numpy(), "blob == NULL")
+
+
+def test_rejected_arguments(hip, device, oracle):
+    dev, copy, _ = _weight(hip, device, oracle, 72, 512, 31)
+    x = activations(40, 512, 35)
+    with pytest.raises(GQHipError) as e:  # a copy that is not 16-byte aligned
+        _run(hip, device, x, dev, copy.blob[8:], None, 72, 512, 0)
+    assert e.value.code == GQ_ERR_MISALIGNED
+    # no streaming layout exists for group size 32 or for 320 input features: a copy cannot be meant
+    packed, scale, bias = group_quantize_compress_numpy(normal_weight(64, 320, 3), 64)
+    odd = tuple(to_dev(a, device) for a in (packed, scale, bias))
+    with pytest.raises(GQHipError) as e:
+        _run(hip, device, activations(40, 320, 36), odd, copy.blob, None, 64, 320, 0)
+    assert e.value.code == GQ_ERR_UNSUPPORTED and "streaming layout" in str(e.value)
+
+
+def test_layer_with_the_copy(hip, device, oracle):
+    """LinearGQ(dim=0) after prepack_for_decode(): prefill batches read the copy, decode batches the
+    variables; the same results as before the copy was made."""
+    from popxl_addons.layers.linear_gq import LinearGQ
+
+    n_out, k_in = 4096, 4096
+    layer = LinearGQ(n_out, bias=True, group_size=64, dim=0)
+    layer.init_variables(k_in, torch.float16, device)
+    (p, s, b), _, w_dec = _weight(hip, device, oracle, n_out, k_in, 31)
+    ob = np.random.default_rng(37).normal(0, 1, (n_out,)).astype(np.float16)
+    v = layer.variables
+    v.weight_compressed.data.copy_(p.reshape(v.weight_compressed.shape))
+    v.weight_decompression_scale.data.copy_(s.reshape(v.weight_decompression_scale.shape))
+    v.weight_decompression_bias.data.copy_(b.reshape(v.weight_decompression_bias.shape))
+    v.bias.data.copy_(to_dev(ob, device))
+    for m_rows in (4, 300):
+        x = activations(m_rows, k_in, 38 + m_rows)
+        before = layer(to_dev(x, device)).cpu().numpy()
+        copy = layer.prepack_for_decode()
+        assert copy.layout == "nk" and layer._decode_copy is copy
+        after = layer(to_dev(x, device)).cpu().numpy()
+        assert_bits_equal(after, before, m_rows)
+        assert_close(after, oracle.np_linear(x, w_dec, ob), m_rows)
+        layer._decode_copy = None
