@@ -766,6 +766,8 @@ def main():
     ap.add_argument("--stack-modes", default="",
                     help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
     ap.add_argument("--stack-batches", default="1,4,8", help="batch sizes of the stack runs")
+    ap.add_argument("--knp-shapes", default="", help="--only knp: decode rows on these weights instead (n_out x k_in, e.g. 4096x20480,28672x4096)")
+    ap.add_argument("--knp-batches", default="1,8", help="decode batches of the knp rows")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
                     help="file for every figure of the run (the stdout line holds a summary); empty: no file")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -868,15 +870,16 @@ def main():
     if args.only in ("kn", "knp", "all"):
         # ... and from the derived copy that a layer keeps after prepack_for_decode(): the kn streaming layout
         extra["linear_knp"] = []
-        for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
-            for m in (1, 8):
+        shapes = [tuple(int(v) for v in s.split("x")) for s in args.knp_shapes.split(",") if s] or [(4096, 4096), (16384, 4096), (4096, 16384)]
+        for n_out, k_in in shapes:
+            for m in [int(v) for v in args.knp_batches.split(",")]:
                 r = bench_linear(hip, device, "gq_linear_knp_act_f16", m, n_out, k_in, 200, 20,
                                  n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_knp_kernel")
                 extra["linear_knp"].append(r)
                 log(f"  kn streaming layout gemv m={m} [{k_in}->{n_out}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
         # prefill batches from the same copy (configuration 4 in the default layout): the MFMA pipeline of the other layout
-        for m in (128, 512, 2048):
+        for m in (() if args.knp_shapes else (128, 512, 2048)):
             r = bench_linear(hip, device, "gq_linear_knp_act_f16", m, 16384, 4096, 60, 5, n_sets=sets_beyond_cache(16384, 4096),
                              kernel="gemm_pipe2_kn_kernel")
             extra["linear_knp"].append(r)
