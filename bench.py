@@ -708,7 +708,7 @@ def headline(result):
     extra = result.get("extra") or {}
     short = {k: extra[k] for k in ("detail_file", "gpu_equals_cpu_baseline_bits", "bench_wall_s") if k in extra}
     if any(k in extra for k in ("gemv", "linear_kn", "gemm")):
-        short["weights"] = "every row rotates over distinct weights of > 600 MB packed bytes in total (n_sets in the detail file)"
+        short["weights"] = "every row rotates over > 600 MB of distinct packed weights"
     for key in ("decompress_transposed", "compress", "compress_f32"):
         if key in extra:
             short[key] = {"us": round(extra[key]["us"], 1), "frac": round(extra[key]["hbm_frac"], 3)}
@@ -717,9 +717,9 @@ def headline(result):
     if "linear_knp" in extra:  # the same shapes in the default layout of LinearGQ ([k_in, n_out]), from the derived copy
         short["c3_gemv_default_layout"] = [_row(r, "hbm_frac") for r in extra["linear_knp"] if r["m"] <= 16]
         short["c4_gemm_default_layout"] = [_row(r, "mfma_frac") for r in extra["linear_knp"] if r["m"] > 16]
-    if "linear_kn" in extra:  # ... and from the three variables as they are (the other batches: in the detail file)
-        short["c3_gemv_default_layout_variables"] = [_row(r, "hbm_frac") for r in extra["linear_kn"] if r["m"] == 1]
-        short["gemm_default_layout_variables"] = [_row(r, "mfma_frac") for r in extra["linear_kn"] if r["m"] > 16]
+    if "gemv_streaming_layout" in extra:  # configuration 3 with the weight's derived copy beside the variables
+        short["c3_gemv_streaming_layout"] = [_row(r, "hbm_frac") for r in extra["gemv_streaming_layout"]]
+    # (the default layout from the three variables as they are, `linear_kn`: in the detail file)
     if "gemm" in extra:  # configuration 4: fraction of the dense fp16 MFMA peak
         short["c4_gemm"] = [_row(r, "mfma_frac") for r in extra["gemm"]]
     if "gemm_streaming_layout" in extra:  # ... the same with the weight's derived copy beside the variables
@@ -852,6 +852,17 @@ def main():
                                  n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_mfma_kernel / gemv_stream_single_kernel")
                 extra["gemv"].append(r)
                 log(f"  gemv m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
+                torch.cuda.empty_cache()
+    if args.only in ("gemv", "all"):
+        # the same rows when the caller also holds the weight's derived copy in the streaming layout (what LinearGQ(dim=0)
+        # does after prepack_for_decode()): the same kernel and the same bits, every load 1 KiB contiguous and read once
+        extra["gemv_streaming_layout"] = []
+        for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
+            for m in (1, 8):
+                r = bench_linear(hip, device, "gq_linear_p_act_f16", m, n_out, k_in, 200, 20,
+                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_mfma_kernel (streaming layout)")
+                extra["gemv_streaming_layout"].append(r)
+                log(f"  gemv, streaming layout m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
     if args.only in ("kn", "all"):
         # the same shapes with the weight stored [k_in, n_out] and grouped along n_out: the default layout of LinearGQ

@@ -157,9 +157,10 @@ int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
  * variables, popxl_addons/layers/linear_gq.py:99-109).  Batches of more than 16 rows that run the
  * pipelined GEMM kernel then read the copy, whose pieces are 512 bytes contiguous where a row of
  * `packed` contributes 32 bytes per step of 64 input features: the same results to the tolerance of
- * the fused paths, 5 - 12 % sooner.  Every other path (m_rows <= 16, passes of the GEMV kernel, shapes
- * outside the pipelined kernel) reads packed, scale and bias as gq_linear_act_ws_f16 does, so these
- * stay required.  blob == NULL: the call is gq_linear_act_ws_f16.
+ * the fused paths, 5 - 12 % sooner; batches of up to 16 rows and passes of the GEMV kernel read it
+ * too (each load 1 KiB contiguous and read once).  The shapes outside those kernels read packed,
+ * scale and bias as gq_linear_act_ws_f16 does, so these stay required.  blob == NULL: the call is
+ * gq_linear_act_ws_f16.
  */
 int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const void *blob, const uint16_t *out_bias, uint16_t *y,
@@ -310,8 +311,9 @@ typedef struct gq_gemv_desc {
  *   gq_gemv_prepacked_bytes  size of the blob in bytes, or a negative GQ_ERR_* code
  *   gq_gemv_prepack_f16      writes the blob (device memory, 16-byte aligned) from packed / scale /
  *                            bias (16-byte aligned) on `stream`
- * An entry of a sequence uses the blob by passing it as `packed` with scale == bias == NULL; such
- * an entry needs m_rows <= 4 and a sequence that runs on the persistent kernel as a whole.
+ * An entry of a sequence uses the blob by passing it as `packed` with scale == bias == NULL (up to
+ * 16 rows; like any entry it joins a run of the persistent kernels up to 4 rows and is a launch of
+ * its own above).  gq_linear_p_act_f16 takes the blob beside the three variables.
  */
 int64_t gq_gemv_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size);
 int gq_gemv_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob,

@@ -186,10 +186,10 @@ int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packe
     workspace = nullptr;
   if (m_rows <= 16)
     return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
-                           (hipStream_t)stream);
+                           (hipStream_t)stream, blob);
   int passes_rc = GQ_OK;
   if (gq::launch_gemv_passes(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation,
-                             workspace != nullptr, (hipStream_t)stream, &passes_rc))
+                             workspace != nullptr, (hipStream_t)stream, &passes_rc, blob))
     return passes_rc;
   return gq::launch_gemm(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation, workspace,
                          (hipStream_t)stream, blob);
@@ -296,11 +296,11 @@ static int gemv_sequence_common(const gq_gemv_desc *descs, const gq_gemv_desc *d
       continue;
     }
     if (blob) {
-      // the weight in the streaming layout: only the persistent kernel reads it
-      if (d.group_size != 64 || d.k_in <= 0 || d.k_in % 512 != 0 || d.m_rows < 1 || d.m_rows > 4 || d.n_out < 1)
+      // the weight in the streaming layout (the persistent kernels up to 4 rows, a launch of the one-shot kernel above)
+      if (d.group_size != 64 || d.k_in <= 0 || d.k_in % 512 != 0 || d.m_rows < 1 || d.m_rows > 16 || d.n_out < 1)
         return gq::fail(GQ_ERR_UNSUPPORTED,
                         "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which needs group_size 64, "
-                        "k_in %% 512 == 0 and 1 <= m_rows <= 4 (got group_size=%d k_in=%d m_rows=%d n_out=%d)",
+                        "k_in %% 512 == 0 and 1 <= m_rows <= 16 (got group_size=%d k_in=%d m_rows=%d n_out=%d)",
                         (long long)i, d.group_size, d.k_in, d.m_rows, d.n_out);
       if (gq::misaligned(d.packed, 16) || gq::misaligned(d.x, 16))
         return gq::fail(GQ_ERR_MISALIGNED, "gq_gemv_sequence_f16: entry %lld: blob and x must be 16-byte aligned",

@@ -47,9 +47,10 @@ __device__ __forceinline__ float apply_activation(float v, int act) {
 // Launchers implemented next to their kernels.
 int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
                       int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed, hipStream_t stream);
+// blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16 (packed, scale, bias may then be NULL)
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream);
+                int64_t group_size, int act, hipStream_t stream, const void *blob = nullptr);
 // workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
 // blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16, which the pipelined kernel then reads
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
@@ -62,7 +63,7 @@ double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_sp
 // nothing launched.
 bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc);
+                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc, const void *blob = nullptr);
 int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                              const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                              int64_t k_in, int64_t group_size, int act, hipStream_t stream);

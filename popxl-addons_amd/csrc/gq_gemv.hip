@@ -39,7 +39,12 @@ namespace {
 //       and 1.9 us of 7.1 at eight on 4096 x 4096.)
 constexpr int gemv_region_bytes(int r, int xm) { return (xm > r ? xm : r) * 1024; }
 
-template <int NWAVES, int R, int GS, bool FULL, int XM>
+// BLOB  `packed` is the weight in the streaming layout of gq_gemv_prepack_f16 (scale and bias are not read;
+//       GS == 64 and FULL): item (row block, chunk) = 4 KiB of codes as [slot][kc][r] 16-byte pieces -- each of
+//       the four loads of a chunk is 1 KiB contiguous, read once -- then the rows' 16 bytes of scales, of biases.
+constexpr int kStreamItemBytes = 4608;
+
+template <int NWAVES, int R, int GS, bool FULL, int XM, bool BLOB = false>
 __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
@@ -58,6 +63,15 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int row = min(((int)blockIdx.x * R + i) * 16 + r, n_out - 1);
+    if constexpr (BLOB) {
+      static_assert(GS == 64 && FULL, "the streaming layout has groups of 64 and whole chunks");
+      const int rb = min((int)blockIdx.x * R + i, ((n_out + 15) >> 4) - 1);  // (the copy pads the last row block)
+      const char *const items = reinterpret_cast<const char *>(packed) + (int64_t)rb * n_chunks * kStreamItemBytes;
+      wrow[i] = reinterpret_cast<const uint4_t *>(items) + lane;
+      srow[i] = reinterpret_cast<const half_t *>(items + 4096 + r * 16);
+      brow[i] = reinterpret_cast<const half_t *>(items + 4352 + r * 16);
+      continue;
+    }
     wrow[i] = packed + (int64_t)row * (k_in >> 5) + kc;
     srow[i] = scale + (int64_t)row * groups_per_row;
     brow[i] = bias + (int64_t)row * groups_per_row;
@@ -93,9 +107,12 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int slot = c * 4 + j;
-        if (FULL || slot < n_slots)
+        if (BLOB)
+          wq[i][j] = __builtin_nontemporal_load(wrow[i] + c * (kStreamItemBytes / 16) + j * 64);
+        else if (FULL || slot < n_slots)
           // (ordinary loads: marked read-once they were 1 - 8 % slower on every shape and batch but
-          // 4096 x 4096, where it makes no difference: 12288 x 4096 at 8 rows 12.5 against 11.3 us)
+          // 4096 x 4096, where it makes no difference: 12288 x 4096 at 8 rows 12.5 against 11.3 us --
+          // a lane's 16 bytes are part of a line that the other slots' loads complete)
           wq[i][j] = *(wrow[i] + slot * 4);
         else
           wq[i][j] = uint4_t{0u, 0u, 0u, 0u};
@@ -106,8 +123,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
         // The dwords that then stand for the absent slots belong to earlier groups of the row: finite
         // numbers, multiplied by codes and x that are zero.
         const int back = (!FULL && c == n_chunks - 1) ? 4 - (n_slots - c * 4) : 0;
-        uint4_t sv = *reinterpret_cast<const uint4_t *>(srow[i] + c * 8 - back * 2);
-        uint4_t bv = *reinterpret_cast<const uint4_t *>(brow[i] + c * 8 - back * 2);
+        uint4_t sv = *reinterpret_cast<const uint4_t *>(srow[i] + (BLOB ? c * (kStreamItemBytes / 2) : c * 8 - back * 2));
+        uint4_t bv = *reinterpret_cast<const uint4_t *>(brow[i] + (BLOB ? c * (kStreamItemBytes / 2) : c * 8 - back * 2));
         if (!FULL) {
           if (back & 1) sv = uint4_t{sv.y, sv.z, sv.w, sv.x}, bv = uint4_t{bv.y, bv.z, bv.w, bv.x};
           if (back & 2) sv = uint4_t{sv.z, sv.w, sv.x, sv.y}, bv = uint4_t{bv.z, bv.w, bv.x, bv.y};
@@ -242,9 +259,16 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 
 }  // namespace
 
+// `blob`: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16 (then group_size is 64 and
+// k_in % 512 == 0); with x and the blob 16-byte aligned the kernels read it and packed, scale, bias may be NULL.
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream) {
+                int64_t group_size, int act, hipStream_t stream, const void *blob) {
+  if (blob && (group_size != 64 || k_in % 512 != 0 || k_in <= 0 || ((uintptr_t)x % 16) != 0 || ((uintptr_t)blob % 16) != 0)) {
+    if (!packed || !scale || !bias)
+      return fail(GQ_ERR_UNSUPPORTED, "a weight in the streaming layout needs group_size 64, k_in %% 512 == 0 and 16-byte aligned x");
+    blob = nullptr;  // (the variables serve)
+  }
   // Weights of 72 Mi elements or more with rows shorter than 8192 features go through the persistent
   // kernel at batches up to 4, as a sequence of one: its pipelined rings beat the one-shot kernel below
   // there (measured at one row: 20480x4096 15.1 -> 13.2 us, 24576x4096 19.7 -> 14.6 us, 32768x4096
@@ -253,9 +277,14 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   // overlap and wins (4096x16384 at one row: 12.0 against 14.5 us; 8192x8192: 13.3 against 14.1).
   const bool large = n_out * k_in >= ((int64_t)72 << 20) && k_in < 8192;
   if (large && m_rows <= 4) {
-    const int rc =
-        launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
+    const int rc = blob ? launch_gemv_streamed(x, m_rows, static_cast<const uint16_t *>(blob), nullptr, nullptr, out_bias, y, n_out,
+                                               k_in, group_size, act, stream)
+                        : launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
     if (rc != GQ_ERR_UNSUPPORTED) return rc;
+  }
+  if (blob) {  // (shape and alignment were checked above: the streaming-layout instantiations of the one-shot kernel)
+    packed = static_cast<const uint16_t *>(blob);
+    scale = bias = nullptr;
   }
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
@@ -284,7 +313,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     const uintptr_t sb_align = (uintptr_t)scale | (uintptr_t)bias;
     // (group 64 with a partial last chunk, e.g. k_in = 11008: the rows of scale / bias are then only
     // 4-byte aligned, which the 16-byte loads take, and the last load reaches back into the chunk before)
-    const int gs_mode = (group_size == 64 && (full || k_in > 512) && sb_align % 16 == 0)
+    const int gs_mode = blob ? 64 : (group_size == 64 && (full || k_in > 512) && sb_align % 16 == 0)
                             ? 64
                             : ((group_size == 128 && full && sb_align % 8 == 0) ? 128 : 0);
     const unsigned blocks = (unsigned)((row_blocks + r - 1) / r);
@@ -292,7 +321,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),                    \
       reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act
-#define GQ_GEMV_LAUNCH(NW, R, GS, FULL, XM)                                                              \
+#define GQ_GEMV_LAUNCH(NW, R, GS, FULL, XM, BLOB)                                                            \
   do {                                                                                                    \
     constexpr int lds_bytes = NW * gemv_region_bytes(R, XM);                                              \
     static_assert(lds_bytes <= 160 * 1024, "LDS budget");                                                \
@@ -303,35 +332,36 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
       if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return GQ_ERR_NO_DEVICE;     \
       if (!configured[dev]) {                                                                             \
         const hipError_t e = hipFuncSetAttribute(                                                         \
-            reinterpret_cast<const void *>(gemv_mfma_kernel<NW, R, GS, FULL, XM>),                        \
+            reinterpret_cast<const void *>(gemv_mfma_kernel<NW, R, GS, FULL, XM, BLOB>),                       \
             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                                       \
         if (e != hipSuccess) return fail((int)e, "hipFuncSetAttribute: %s", hipGetErrorString(e));        \
         configured[dev] = true;                                                                           \
       }                                                                                                   \
     }                                                                                                     \
-    gemv_mfma_kernel<NW, R, GS, FULL, XM><<<dim3(blocks), dim3(NW * 64), lds_bytes, stream>>>(GQ_GEMV_ARGS); \
+    gemv_mfma_kernel<NW, R, GS, FULL, XM, BLOB><<<dim3(blocks), dim3(NW * 64), lds_bytes, stream>>>(GQ_GEMV_ARGS); \
   } while (0)
-#define GQ_GEMV_BY_R(NW, GS, FULL, XM)                      \
-  do {                                                      \
-    if (r == 4) GQ_GEMV_LAUNCH(NW, 4, GS, FULL, XM);        \
-    else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL, XM);   \
-    else GQ_GEMV_LAUNCH(NW, 1, GS, FULL, XM);               \
+#define GQ_GEMV_BY_R(NW, GS, FULL, XM, BLOB)                      \
+  do {                                                            \
+    if (r == 4) GQ_GEMV_LAUNCH(NW, 4, GS, FULL, XM, BLOB);        \
+    else if (r == 2) GQ_GEMV_LAUNCH(NW, 2, GS, FULL, XM, BLOB);   \
+    else GQ_GEMV_LAUNCH(NW, 1, GS, FULL, XM, BLOB);               \
   } while (0)
     // x through LDS, one load instruction per batch row and chunk (the rows of x are 16-byte aligned:
     // k_in % 128 == 0), on eight waves whatever the length of the rows (measured on 4096 x 16384:
     // 16 waves are no faster with x staged; without, eight rows took 20.1 us against 14.7 us)
-#define GQ_GEMV_BY_M(GS, FULL)                              \
-  do {                                                      \
-    if (m_rows == 1) GQ_GEMV_BY_R(8, GS, FULL, 1);          \
-    else if (m_rows <= 4) GQ_GEMV_BY_R(8, GS, FULL, 4);     \
-    else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, FULL, 8);     \
-    else GQ_GEMV_BY_R(8, GS, FULL, 16);                     \
+#define GQ_GEMV_BY_M(GS, FULL, BLOB)                              \
+  do {                                                            \
+    if (m_rows == 1) GQ_GEMV_BY_R(8, GS, FULL, 1, BLOB);          \
+    else if (m_rows <= 4) GQ_GEMV_BY_R(8, GS, FULL, 4, BLOB);     \
+    else if (m_rows <= 8) GQ_GEMV_BY_R(8, GS, FULL, 8, BLOB);     \
+    else GQ_GEMV_BY_R(8, GS, FULL, 16, BLOB);                     \
   } while (0)
-    if (gs_mode == 64 && full) GQ_GEMV_BY_M(64, true);
-    else if (gs_mode == 64) GQ_GEMV_BY_M(64, false);
-    else if (gs_mode == 128) GQ_GEMV_BY_M(128, true);
-    else if (full) GQ_GEMV_BY_M(0, true);
-    else GQ_GEMV_BY_M(0, false);  // (a last chunk of 128, 256 or 384 features, e.g. k_in = 11008)
+    if (blob) GQ_GEMV_BY_M(64, true, true);
+    else if (gs_mode == 64 && full) GQ_GEMV_BY_M(64, true, false);
+    else if (gs_mode == 64) GQ_GEMV_BY_M(64, false, false);
+    else if (gs_mode == 128) GQ_GEMV_BY_M(128, true, false);
+    else if (full) GQ_GEMV_BY_M(0, true, false);
+    else GQ_GEMV_BY_M(0, false, false);  // (a last chunk of 128, 256 or 384 features, e.g. k_in = 11008)
 #undef GQ_GEMV_BY_M
 #undef GQ_GEMV_BY_R
 #undef GQ_GEMV_LAUNCH
@@ -354,7 +384,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 // rows 69.7 against 117.1, 16384 x 4096 at 32 rows 25.4 against 34.1 (and 38.0 against 35.2 at 48 rows).
 bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc) {
+                        int64_t group_size, int act, bool gemm_may_split, hipStream_t stream, int *rc, const void *blob) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)packed % 16) == 0;
@@ -368,7 +398,7 @@ bool launch_gemv_passes(const uint16_t *x, int64_t m_rows, const uint16_t *packe
   if ((double)passes * t_pass >= t_gemm) return false;
   for (int64_t m0 = 0; m0 < m_rows; m0 += 16) {
     const int64_t m = m_rows - m0 < 16 ? m_rows - m0 : 16;
-    *rc = launch_gemv(x + m0 * k_in, m, packed, scale, bias, out_bias, y + m0 * n_out, n_out, k_in, group_size, act, stream);
+    *rc = launch_gemv(x + m0 * k_in, m, packed, scale, bias, out_bias, y + m0 * n_out, n_out, k_in, group_size, act, stream, blob);
     if (*rc != GQ_OK) return true;
   }
   return true;

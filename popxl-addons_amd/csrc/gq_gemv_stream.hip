@@ -1029,10 +1029,12 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
     if (persistent(i)) {
       any_persistent = true;
     } else if (prepacked(host[i]) && !(host[i].activation & GQ_DESC_KN_LAYOUT)) {
-      return fail(GQ_ERR_UNSUPPORTED,
-                  "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which only the persistent kernel "
-                  "reads, but its shape is outside that kernel (group 64, k_in %% 512 == 0, m_rows <= 4, 16-byte aligned)",
-                  (long long)i);
+      // (a launch of its own: batches of 5 to 16 rows; the one-shot kernel reads the streaming layout too)
+      const gq_gemv_desc &d = host[i];
+      if (!(d.group_size == 64 && d.k_in > 0 && d.k_in % 512 == 0 && ((uintptr_t)d.x % 16) == 0 && ((uintptr_t)d.packed % 16) == 0))
+        return fail(GQ_ERR_UNSUPPORTED,
+                    "gq_gemv_sequence_f16: entry %lld is in the streaming layout, which needs group 64, k_in %% 512 == 0 "
+                    "and 16-byte aligned x and weight", (long long)i);
     }
   }
   int dev = 0, grid = 0;
@@ -1078,7 +1080,7 @@ int launch_gemv_sequence(const gq_gemv_desc *host, const gq_gemv_desc *device, i
       const int rc = (d.activation & GQ_DESC_KN_LAYOUT)
                          ? launch_gemv_knp(d.x, d.m_rows, d.packed, d.out_bias, d.y, d.n_out, d.k_in, act, stream)
                          : launch_gemv(d.x, d.m_rows, d.packed, d.scale, d.bias, d.out_bias, d.y, d.n_out, d.k_in,
-                                       d.group_size, act, stream);
+                                       d.group_size, act, stream, prepacked(d) ? d.packed : nullptr);
       if (rc != GQ_OK) return rc;
       ++first;
       continue;

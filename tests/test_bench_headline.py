@@ -40,6 +40,7 @@ def full_detail():
         "decompress_transposed": {"rows": 4096, "cols": 16384, "us": 26.3456789, "gbs": 6531.123456, "hbm_frac": 0.81612345,
                                   "roofline": bench.hbm_roofline("decompress_transposed_tile_kernel", 171966464.0, 0.0263)},
         "gemv": [_linear_row(m, n, k, "gemv_mfma_kernel / gemv_stream_single_kernel", "hbm") for n, k in shapes for m in (1, 8)],
+        "gemv_streaming_layout": [_linear_row(m, n, k, "gemv_mfma_kernel (streaming layout)", "hbm") for n, k in shapes for m in (1, 8)],
         "linear_kn": [_linear_row(m, n, k, "gemv_kn_kernel", "hbm") for n, k in shapes for m in (1, 8)]
         + [_linear_row(128, 16384, 4096, "gemm_kn_tile_kernel", "mfma")],
         "linear_knp": [_linear_row(m, n, k, "gemv_knp_kernel", "hbm") for n, k in shapes for m in (1, 8)]
@@ -90,7 +91,8 @@ def test_headline_is_short_and_complete():
     assert "legs" not in back["cpu_baseline"]
     # one short record per benchmark shape of configurations 3, 4 and 5
     assert len(back["extra"]["c3_gemv"]) == 6 and len(back["extra"]["c3_gemv_default_layout"]) == 6
-    assert len(back["extra"]["c3_gemv_default_layout_variables"]) == 3  # (batch 1 only: the rest is in the detail file)
+    assert len(back["extra"]["c3_gemv_streaming_layout"]) == 6
+    assert "c3_gemv_default_layout_variables" not in back["extra"]  # (the kernels on the default layout's variables: detail file only)
     assert [r["m"] for r in back["extra"]["c4_gemm"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c4_gemm_default_layout"]] == [128, 512, 2048]
     assert [r["m"] for r in back["extra"]["c4_gemm_streaming_layout"]] == [128, 512, 2048]

@@ -518,12 +518,22 @@ def test_gemv_sequence_streaming_layout(hip, device, oracle, m_rows, chained):
     top = want.float().abs().max().item()
     assert (y.float() - want.float()).abs().max().item() <= 1.5e-3 * top
     assert_close(y32.cpu().numpy(), oracle.np_linear(x32, oracle.np_decompress(p32, s32, b32)))
-    # what stays refused: a blob whose shape is outside the persistent kernel (more than four batch rows)
-    tall = GemvSequence(device)
-    x5 = to_dev(activations(5, x.shape[1], 2), device)
-    tall.add(x5, prepack_gemv(packed, scale, bias), None, None, torch.empty((5, packed.shape[0]), dtype=torch.float16, device=device))
-    with pytest.raises(GQHipError) as e:
+    # more than four batch rows: outside the persistent kernels, the blob's entry is a launch of the one-shot kernel,
+    # which reads the streaming layout as well; what stays refused is more than sixteen
+    w_dec = oracle.np_decompress(*(a.cpu().numpy() for a in (packed, scale, bias)))
+    for rows in (5, 16):
+        tall = GemvSequence(device)
+        x_tall = activations(rows, x.shape[1], 2)
+        y_tall = torch.full((rows, packed.shape[0]), float("nan"), dtype=torch.float16, device=device)
+        tall.add(to_dev(x_tall, device), prepack_gemv(packed, scale, bias), None, None, y_tall, ob)
         tall.run()
+        tall.check()
+        assert_close(y_tall.cpu().numpy(), oracle.np_linear(x_tall, w_dec, None if ob is None else ob.cpu().numpy()), rows)
+    too_tall = GemvSequence(device)
+    x17 = to_dev(activations(17, x.shape[1], 2), device)
+    too_tall.add(x17, prepack_gemv(packed, scale, bias), None, None, torch.empty((17, packed.shape[0]), dtype=torch.float16, device=device))
+    with pytest.raises(GQHipError) as e:
+        too_tall.run()
     assert "streaming layout" in str(e.value)
 
 

@@ -1,8 +1,8 @@
 """gq_linear_p_act_f16: the fused matmul for weights grouped along the input features (LinearGQ with
 dim=0) when the caller also holds the derived copy in the streaming layout (gq_gemv_prepack_f16).
-The pipelined GEMM kernel then reads the copy; the arithmetic is that of gq_linear_act_ws_f16 on the
-three variables, so the results are the oracle's to the tolerance of the fused paths AND equal to
-that entry point's bit for bit."""
+The one-shot GEMV kernel and the pipelined GEMM kernel then read the copy; the arithmetic is that of
+gq_linear_act_ws_f16 on the three variables, so the results are the oracle's to the tolerance of the
+fused paths AND equal to that entry point's bit for bit."""
 import numpy as np
 import pytest
 import torch
@@ -50,13 +50,28 @@ def test_benchmark_prefill_batches(hip, device, oracle, m_rows):
     assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 0), "against the variables")
 
 
+@pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (16384, 4096), (4096, 16384), (28672, 4096), (1000, 1536), (16, 512)])
+@pytest.mark.parametrize("m_rows", [1, 3, 4, 8, 16])
+def test_decode_batches(hip, device, oracle, n_out, k_in, m_rows):
+    """Up to 16 rows the one-shot GEMV kernel reads the copy (every load 1 KiB contiguous, read once) -- on the
+    widest weight at up to 4 rows the persistent kernel as a sequence of one: the oracle's result, and the bits
+    of the same call on the variables where the same kernel runs."""
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 41)
+    x = activations(m_rows, k_in, 42 + m_rows)
+    ob = np.random.default_rng(43).normal(0, 1, (n_out,)).astype(np.float16) if m_rows % 2 else None
+    y = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 1)
+    assert_close(y, oracle.np_linear(x, w_dec, ob, "relu"), (n_out, k_in, m_rows))
+    if not (n_out == 28672 and m_rows <= 4):
+        assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 1), "against the variables")
+
+
 @pytest.mark.parametrize("n_out,k_in,m_rows", [(4096, 4096, 300), (4096, 16384, 128), (4104, 512, 300), (8200, 1024, 777),
                                                (4104, 1536, 2060), (1000, 4096, 40), (72, 512, 33), (16384, 4096, 64),
                                                (4096, 4096, 17), (4096, 4096, 8)])
 def test_shapes_with_and_without_workspace(hip, device, oracle, n_out, k_in, m_rows):
     """Ragged tiles and row blocks (n_out not a multiple of 16: the copy pads the last block), K divided
     over workgroups through the workspace, the 64 x 64 tiles, batches that run as passes of the GEMV
-    kernel or as one GEMV (those read the variables whether the copy is there or not), an activation."""
+    kernel or as one GEMV, an activation."""
     dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 31)
     x = activations(m_rows, k_in, 32)
     ob = np.random.default_rng(33).normal(0, 1, (n_out,)).astype(np.float16)
