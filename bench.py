@@ -669,6 +669,77 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         if not worst <= 2e-3 or results[mode]["status"] != 0 or not worst_oracle <= 1e-2:
             raise SystemExit(f"bench.py: stack mode {mode} (m={m_rows}) is wrong: error {worst} against single calls, "
                              f"{worst_oracle} against the oracle, status {results[mode]['status']}")
+    # (3) the decoder's data flow with two launches per layer through the layer's entry point, gq_linear_p_act_f16 with the
+    # derived copy beside the variables, replayed from a HIP graph: what serves batches of more than four rows, which the
+    # persistent kernels do not take.  The weights of the two-entry schedule above: up | v | q | k stacked along the
+    # outputs, then the joint output product [down | o] (scaled by 0.27: no normalisation layers here).
+    mode = "streaming_layout_two_entries_graph"
+    if modes is None or mode in modes:
+        two = []
+        for layer in range(n_layers):
+            q, k, v, o, up, down = (mats[layer * 6 + role][2:] for role in range(6))
+            first = tuple(torch.cat([up[part], v[part], q[part], k[part]], dim=0).contiguous() for part in range(3))
+            out = [torch.cat([down[part], o[part]], dim=1).contiguous() for part in range(3)]
+            out = (out[0], (out[1].float() * 0.27).to(torch.float16), (out[2].float() * 0.27).to(torch.float16))
+            two.append((first, hip.prepack_gemv(*first), out, hip.prepack_gemv(*out)))
+        torch.cuda.synchronize()
+        wide = torch.empty((m_rows, ffn + 3 * hidden), dtype=torch.float16, device=device)
+        h_out = [torch.empty((m_rows, hidden), dtype=torch.float16, device=device) for _ in range(2)]
+        # (more than one row: x of the joint product is gathered by a copy, which stands for the attention and
+        # activation kernels that a model has between the two launches anyway)
+        joint_x = wide if m_rows == 1 else torch.empty((m_rows, ffn + hidden), dtype=torch.float16, device=device)
+
+        def layer_entry(stream, x, variables, copy, y):
+            hip.call("gq_linear_p_act_f16", x.data_ptr(), m_rows, *(t.data_ptr() for t in variables), copy.blob.data_ptr(), 0,
+                     y.data_ptr(), copy.n_out, copy.k_in, GROUP, 0, 0, 0, stream)
+
+        def one_pass_two(stream):
+            h = h0_joint
+            for layer in range(n_layers):
+                first, first_copy, out, out_copy = two[layer]
+                layer_entry(stream, h, first, first_copy, wide)
+                if m_rows > 1:
+                    joint_x.copy_(wide[:, : ffn + hidden])
+                h = h_out[layer % 2]
+                layer_entry(stream, joint_x, out, out_copy, h)
+
+        one_pass_two(stream_handle())
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            one_pass_two(stream_handle())
+        ms = time_launches(lambda _: graph.replay(), passes, warmup)
+        torch.cuda.synchronize()
+        kernel = "gemv_mfma_kernel (streaming layout; 56 launches)" if m_rows > 4 else "gemv_stream_single_kernel / gemv_mfma_kernel (streaming layout; 56 launches)"
+        results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
+                         "status": 0, "roofline": hbm_roofline(kernel, w_bytes, ms)}
+        # the last layer's two results against single calls on the variables (and the oracle, when a test hands it over)
+        worst, worst_oracle = 0.0, 0.0
+        h_last = h_out[(n_layers - 2) % 2]
+        first, _, out, _ = two[n_layers - 1]
+        # (at one row joint_x IS the wide result: the product's x is its first ffn + hidden values, not all of them)
+        for x_in, (p, s_, b), y in ((h_last, first, wide), (joint_x[:, : ffn + hidden], out, h_out[(n_layers - 1) % 2])):
+            assert x_in.is_contiguous() and x_in.shape[1] * 2 == p.shape[1] * p.shape[2] * 8 and y.shape[1] == p.shape[0]
+            ref = torch.empty_like(y)
+            hip.call("gq_gemv_f16", x_in.data_ptr(), m_rows, p.data_ptr(), s_.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),
+                     y.shape[1], x_in.shape[1], GROUP, stream_handle())
+            torch.cuda.synchronize()
+            err = ((y.float() - ref.float()).abs().max() / ref.float().abs().max()).item()
+            worst = err if not (err <= worst) else worst
+            if oracle is not None:
+                import numpy as np
+
+                ref64 = oracle.np_linear(x_in.cpu().numpy(), oracle.np_decompress(*(t.cpu().numpy() for t in (p, s_, b))))
+                err = float(np.abs(y.cpu().numpy().astype(np.float64) - ref64).max() / np.abs(ref64).max())
+                worst_oracle = err if not (err <= worst_oracle) else worst_oracle
+        results[mode]["max_error_vs_single_call"] = worst
+        if oracle is not None:
+            results[mode]["max_error_vs_oracle"] = worst_oracle
+        if not worst <= 2e-3 or not worst_oracle <= 1e-2:
+            raise SystemExit(f"bench.py: stack mode {mode} (m={m_rows}) is wrong: error {worst} against single calls, "
+                             f"{worst_oracle} against the oracle")
+        del graph, two
+        torch.cuda.empty_cache()
     return results
 
 
@@ -676,7 +747,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
 HEADLINE_LIMIT = 4096  # bytes: the final stdout line must stay a line that a log capture keeps whole
 
 # the decoder schedules of the stack, best first where several ran: what "decoder" means in the headline
-DECODER_MODES = ("sequence_decoder_data_flow_two_entries_streaming_layout", "sequence_decoder_data_flow_joint_output_streaming_layout",
+DECODER_MODES = ("streaming_layout_two_entries_graph",
+                 "sequence_decoder_data_flow_two_entries_streaming_layout", "sequence_decoder_data_flow_joint_output_streaming_layout",
                  "sequence_decoder_data_flow_streaming_layout", "sequence_decoder_data_flow",
                  "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout", "sequence_parallel_block_fused_qkv_ffn_first")
 
@@ -935,7 +1007,7 @@ def main():
             # (more than four batch rows: outside the persistent kernels, every entry is a launch of its own -- the
             # graph of single launches, one sequence, and the default layout's graphs say what there is to say)
             big = ("per_launch_graph", "sequence_parallel_block_fused_qkv_ffn_first", "default_layout_graph",
-                   "default_layout_two_entries_graph")
+                   "default_layout_two_entries_graph", "streaming_layout_two_entries_graph")
             r = bench_stack(hip, device, m, passes=100, warmup=40, modes=modes if modes or m <= 4 else big)
             extra["stack"].append(r)
             for mode, v in r.items():

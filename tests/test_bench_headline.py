@@ -23,7 +23,8 @@ def _stack(m):
              "sequence_parallel_block_fused_qkv_ffn_first", "sequence_parallel_block_fused_qkv_ffn_first_streaming_layout",
              "sequence_decoder_data_flow", "sequence_decoder_data_flow_streaming_layout",
              "sequence_decoder_data_flow_joint_output_streaming_layout", "sequence_decoder_data_flow_two_entries_streaming_layout",
-             "sequence_no_waits", "sequence_no_waits_streaming_layout", "default_layout_graph", "default_layout_sequence")
+             "sequence_no_waits", "sequence_no_waits_streaming_layout", "default_layout_graph", "default_layout_sequence",
+             "streaming_layout_two_entries_graph")
     r = {"m": m, "entries": 168, "weight_bytes": 3170893824.0}
     for i, mode in enumerate(modes):
         r[mode] = {"us_per_pass": 1234.56789 - i, "weight_gbs": 2568.123456, "hbm_frac": 0.32101234, "status": 0, "waits_per_pass": 84,
@@ -99,7 +100,7 @@ def test_headline_is_short_and_complete():
     assert [r["m"] for r in back["extra"]["c5_stack"]] == [1, 4, 8, 16]
     for r in back["extra"]["c5_stack"]:
         assert set(r) >= {"decoder", "no_waits", "per_launch_graph"}
-        assert r["decoder"]["schedule"] == "decoder_data_flow_two_entries_streaming_layout"  # (the fastest of the made-up rows)
+        assert r["decoder"]["schedule"] == "streaming_layout_two_entries_graph"  # (the fastest of the made-up rows)
 
 
 def test_emit_prints_the_headline_last(tmp_path, capsys):

@@ -1014,6 +1014,17 @@ def test_benchmark_stack_28_layers_batch_4_against_oracle(hip, device, oracle):
     torch.cuda.empty_cache()
 
 
+def test_benchmark_stack_28_layers_batch_8_against_oracle(hip, device, oracle):
+    """Eight batch rows, which the persistent kernels do not take: the two launches per layer through the
+    layer's entry point (the one-shot kernel on the weights' streaming-layout copies), as bench.py times them."""
+    import bench
+
+    modes = ("streaming_layout_two_entries_graph",)
+    r = bench.bench_stack(hip, device, 8, passes=2, warmup=1, modes=modes, oracle=oracle)
+    assert r[modes[0]]["max_error_vs_oracle"] <= REGRESSION_TOL and r[modes[0]]["max_error_vs_single_call"] <= REGRESSION_TOL, r[modes[0]]
+    torch.cuda.empty_cache()
+
+
 def _chained_streaming_case(hip, device, oracle, shapes, seed):
     """Chained entries at one batch row, every weight in the streaming layout: (entries, oracle results)."""
     from popxl_addons._gq_hip import prepack_gemv
