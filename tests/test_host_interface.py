@@ -136,7 +136,7 @@ def test_abi_version_and_error_text_without_gpu():
         _gq_hip.call("gq_gemv_prepack_f16", 16, 16, 8, 16, 64, 512, 64, None)
     assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED
     desc["ptrs"] = [[16, 16, 16, 16, 0, 16], [16, 16, 0, 0, 0, 16]]  # entry 1: scale == bias == NULL
-    desc["ints"] = [[1, 8, 512, 64, 0, 0], [5, 8, 512, 64, 1, 0]]
+    desc["ints"] = [[1, 8, 512, 64, 0, 0], [17, 8, 512, 64, 1, 0]]  # (more than 16 rows)
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_gemv_sequence_f16", desc.ctypes.data, 16, 2, None, None)
     assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "streaming layout" in str(e.value)
