@@ -9,7 +9,7 @@ device-side packer that the tests hold bit-identical to the numpy packer).  Inpu
 HBM before the timed region; buffer sets are rotated so that the working set (4 x 172 MB) does not
 fit the 256 MB last-level cache.  The fused GEMV / GEMM / layer-stack measurements of the other
 configurations are summarised in the same JSON line under "extra" (one short record per shape);
-every figure of the run goes to the detail file (default gpurun_out/bench_detail.json) and to stderr.
+every figure of the run goes to the detail file (--detail) and to stderr.
 
 The LAST line on stdout is the one JSON line (under 4 KB); progress goes to stderr.
 """
