@@ -297,6 +297,11 @@ __device__ __forceinline__ void dequant_piece_kn(int piece, uint32_t word, uint4
 // take the places in the wave's ring slot that the 32 scale (bias) dwords of the other layout take;
 // a lane reads the 16 bytes of its step's eight input features from them (all lanes of a half-wave
 // the same: a broadcast), one step ahead of the expansion that uses them.
+// BLOB: `packed` is the weight in the streaming layout of the other layout (groups along the input features;
+// gq_gemv_stream.hip): the same ring slots and arithmetic as from the three variables, but lane (n, h) finds its
+// 16 bytes of K tile T at
+//   item (n / 16, T / 8) + 1024 ((T / 2) % 4) + 512 (T % 2) + 256 h + 16 (n % 16)        (items of 4608 bytes),
+// and the dword with the row's scales (biases) of groups T and T ^ 1 at item + 4096 (4352) + 16 (n % 16) + 4 ((T % 8) / 2).
 template <int WM, int WN, int FM, int FN, int XS, int KS, bool KN = false, bool BLOB = false>
 __device__ __forceinline__ void gemm_pipe2_body(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
