@@ -158,9 +158,11 @@ int gq_linear_act_ws_f16(const uint16_t *x, int64_t m_rows, const uint16_t *pack
  * pipelined GEMM kernel then read the copy, whose pieces are 512 bytes contiguous where a row of
  * `packed` contributes 32 bytes per step of 64 input features: the same results to the tolerance of
  * the fused paths, 5 - 12 % sooner; batches of up to 16 rows and passes of the GEMV kernel read it
- * too (each load 1 KiB contiguous and read once).  The shapes outside those kernels read packed,
- * scale and bias as gq_linear_act_ws_f16 does, so these stay required.  blob == NULL: the call is
- * gq_linear_act_ws_f16.
+ * too (each load 1 KiB contiguous and read once).  Only a call whose x is not 16-byte aligned reads
+ * packed, scale and bias (the kernels of gq_linear_act_ws_f16 for such an x): a caller whose x is
+ * aligned may keep the copy alone and pass all three as NULL (one of them NULL and another not is
+ * GQ_ERR_NULL_POINTER; all three NULL with a misaligned x is GQ_ERR_MISALIGNED).  blob == NULL: the
+ * call is gq_linear_act_ws_f16.
  */
 int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                         const uint16_t *bias, const void *blob, const uint16_t *out_bias, uint16_t *y,

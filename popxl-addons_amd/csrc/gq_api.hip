@@ -170,8 +170,12 @@ int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packe
                         const uint16_t *bias, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                         int64_t k_in, int64_t group_size, int32_t activation, void *workspace, int64_t workspace_bytes,
                         void *stream) {
-  const int rc = gq::check_linear_args("gq_linear_act_f16", x, m_rows, packed, scale, bias, out_bias, y, n_out,
-                                       k_in, group_size);
+  // With the copy, packed, scale and bias may all be NULL (a caller that keeps only the copy): every kernel then reads
+  // the copy, which takes a 16-byte aligned x.  (The copy stands in for them in the checks shared with the other entry points.)
+  const bool only_blob = blob && !packed && !scale && !bias;
+  const uint16_t *const stand_in = static_cast<const uint16_t *>(blob);
+  const int rc = gq::check_linear_args("gq_linear_act_f16", x, m_rows, only_blob ? stand_in : packed, only_blob ? stand_in : scale,
+                                       only_blob ? stand_in : bias, out_bias, y, n_out, k_in, group_size);
   if (rc <= 0) return rc;
   if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_act_f16: unknown activation %d", (int)activation);
@@ -179,6 +183,8 @@ int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packe
     const int64_t blob_bytes = gq_gemv_prepacked_bytes(n_out, k_in, group_size);
     if (blob_bytes < 0) return (int)blob_bytes;  // (no streaming layout for this shape: the message is set)
     if (gq::misaligned(blob, 16)) return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_p_act_f16: blob must be 16-byte aligned");
+    if (only_blob && gq::misaligned(x, 16))
+      return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_p_act_f16: without packed, scale and bias, x must be 16-byte aligned");
   }
   // the workspace is an option: one that is missing, misaligned or too small is not used
   if (m_rows <= 16 || !workspace || gq::misaligned(workspace, 16) ||

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from gq_testlib import activations, assert_bits_equal, normal_weight, to_dev
-from popxl_addons._gq_hip import GQ_ERR_MISALIGNED, GQ_ERR_UNSUPPORTED, GQHipError
+from popxl_addons._gq_hip import GQ_ERR_MISALIGNED, GQ_ERR_NULL_POINTER, GQ_ERR_UNSUPPORTED, GQHipError
 from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy
 from test_gpu_fused import assert_close
 
@@ -85,6 +85,28 @@ def test_shapes_with_and_without_workspace(hip, device, oracle, n_out, k_in, m_r
         assert not ws[:16384].any(), "arrival counters must be back at zero"
 
 
+@pytest.mark.parametrize("n_out,k_in,m_rows", [(4096, 4096, 1), (4096, 16384, 8), (28672, 4096, 2), (1000, 1536, 16), (4096, 4096, 40),
+                                               (4096, 16384, 128), (4104, 1536, 2060), (16384, 4096, 512)])
+def test_the_copy_alone(hip, device, oracle, n_out, k_in, m_rows):
+    """packed, scale and bias NULL: a caller that keeps only the copy.  Every kernel reads the copy (one GEMV,
+    passes of the GEMV kernel, the GEMM kernel with and without K divided over workgroups): the bits of the
+    call that also hands over the variables."""
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 41 if n_out in (28672, 1000) else 31)  # (weights other tests made)
+    x = activations(m_rows, k_in, 52)
+    ob = np.random.default_rng(53).normal(0, 1, (n_out,)).astype(np.float16)
+    need = hip.load().gq_gemm_workspace_bytes(m_rows, n_out, k_in, 64)
+    ws = torch.zeros(max(need, 16384), dtype=torch.uint8, device=device)
+    for workspace in (None, ws):
+        xd, od = to_dev(x, device), to_dev(ob, device)
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        hip.call("gq_linear_p_act_f16", xd.data_ptr(), m_rows, 0, 0, 0, copy.blob.data_ptr(), od.data_ptr(), y.data_ptr(), n_out, k_in,
+                 64, 0, 0 if workspace is None else workspace.data_ptr(), 0 if workspace is None else workspace.numel(),
+                 torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert_close(y.cpu().numpy(), oracle.np_linear(x, w_dec, ob), (n_out, k_in, m_rows))
+        assert_bits_equal(y.cpu().numpy(), _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 0, workspace), "with the variables")
+
+
 def test_without_the_copy_it_is_the_workspace_entry_point(hip, device, oracle):
     n_out, k_in, m_rows = 4096, 4096, 256
     dev, _, _ = _weight(hip, device, oracle, n_out, k_in, 31)
@@ -109,6 +131,17 @@ def test_rejected_arguments(hip, device, oracle):
     with pytest.raises(GQHipError) as e:
         _run(hip, device, activations(40, 320, 36), odd, copy.blob, None, 64, 320, 0)
     assert e.value.code == GQ_ERR_UNSUPPORTED and "streaming layout" in str(e.value)
+    # the copy alone takes a 16-byte aligned x; some of the variables without the others are an error
+    xd = to_dev(activations(41, 512, 37), device)
+    y = torch.empty((40, 72), dtype=torch.float16, device=device)
+    stream = torch.cuda.current_stream().cuda_stream
+    with pytest.raises(GQHipError) as e:
+        hip.call("gq_linear_p_act_f16", xd.data_ptr() + 2, 40, 0, 0, 0, copy.blob.data_ptr(), 0, y.data_ptr(), 72, 512, 64, 0, 0, 0, stream)
+    assert e.value.code == GQ_ERR_MISALIGNED and "16-byte" in str(e.value)
+    with pytest.raises(GQHipError) as e:
+        hip.call("gq_linear_p_act_f16", xd.data_ptr(), 40, 0, dev[1].data_ptr(), dev[2].data_ptr(), copy.blob.data_ptr(), 0, y.data_ptr(),
+                 72, 512, 64, 0, 0, 0, stream)
+    assert e.value.code == GQ_ERR_NULL_POINTER
 
 
 def test_layer_with_the_copy(hip, device, oracle):

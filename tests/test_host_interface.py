@@ -61,6 +61,16 @@ def test_abi_version_and_error_text_without_gpu():
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_f16", 16, 1, 16, 16, 16, 0, 16, 8, 64, 6, None)  # group_size % 4
     assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
+    # the layer's entry with the weight's streaming-layout copy: the copy alone (packed, scale, bias NULL) takes an aligned x
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_p_act_f16", 18, 1, 0, 0, 0, 16, 0, 16, 8, 512, 64, 0, None, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED and "16-byte" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_p_act_f16", 16, 1, 0, 16, 16, 16, 0, 16, 8, 512, 64, 0, None, 0, None)  # packed NULL, scale and bias not
+    assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_p_act_f16", 16, 1, 16, 16, 16, 16, 0, 16, 8, 448, 64, 0, None, 0, None)  # no copy exists for k_in = 448
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "512" in str(e.value)
     # the [k_in, n_out] layout: its own argument rules and the workspace contract
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 96, 64, 64, 0, None, 0, None)  # 96 % 64 != 0
