@@ -166,3 +166,5 @@ def load_layer(checkpoint_dir: str, prefix: str, layer, report_missing: str = "e
             else:
                 t = torch.from_numpy(host)
         var.data.copy_(t.to(var.data.device))
+    if arrays and getattr(layer, "_decode_copy", None) is not None:
+        layer.prepack_for_decode()  # (a derived copy of the variables: make it again)

@@ -186,6 +186,38 @@ def test_checkpoint_round_trip_on_device(hip, device, dim, tmp_path):
     assert_bits_equal(restored(x).cpu().numpy(), y.cpu().numpy())
 
 
+@pytest.mark.parametrize("dim", [0, -1])
+def test_checkpoint_into_a_layer_with_a_derived_copy(hip, device, dim, tmp_path):
+    """A layer that keeps the streaming-layout copy of its weight (prepack_for_decode) and is then loaded from
+    disk serves the loaded weight, at decode and at prefill batches: the copy is made again."""
+    from popxl_addons import checkpoint
+
+    in_features, out_features, group_size = 512, 512, 64
+    layers, outputs = [], []
+    x = {m: torch.randn((m, in_features), device=device, dtype=torch.float16) for m in (3, 70)}
+    for seed in (1, 2):
+        torch.manual_seed(seed)
+        nn_layer = torch.nn.Linear(in_features, out_features)
+        layer = LinearGQ(out_features, bias=True, group_size=group_size, dim=dim)
+        variables = layer.init_variables(in_features, torch.float16, device)
+        layer.load_weights(LinearGQ.torch_mapping(variables, nn_layer, dtype=torch.float16, group_size=group_size, dim=dim))
+        layers.append(layer)
+        outputs.append({m: layer(x[m]).cpu().numpy() for m in x})
+    assert not np.array_equal(outputs[0][3], outputs[1][3])
+    checkpoint.save_layer(str(tmp_path), "block.proj", layers[1])
+    layers[0].prepack_for_decode()
+    stale = layers[0]._decode_copy
+    checkpoint.load_layer(str(tmp_path), "block.proj", layers[0])
+    assert layers[0]._decode_copy is not None and layers[0]._decode_copy is not stale
+    for m in x:
+        got = layers[0](x[m]).cpu().numpy()
+        if dim == 0:
+            assert_bits_equal(got, outputs[1][m], m)  # (the kernels on the copy give the bits of the kernels on the variables)
+        else:
+            err = np.abs(got.astype(np.float32) - outputs[1][m].astype(np.float32)).max() / np.abs(outputs[1][m].astype(np.float32)).max()
+            assert err <= 2e-3, (m, err)  # (another kernel reads the default layout's copy: a few roundings apart)
+
+
 @pytest.mark.parametrize("batch", [1, 4, 40])
 def test_fused_qkv_equals_separate_projections(hip, device, batch):
     """Q, K and V read the same activations: stacking their variables gives one kernel pass whose
