@@ -18,15 +18,23 @@ from test_gpu_fused import assert_close
 pytestmark = pytest.mark.gpu
 
 
+_CASE_WEIGHTS = {}
+
+
 def _case(oracle, n_out, k_in, gs, m_rows, seed, with_bias, activation=None):
     """Weight [k_in, n_out] grouped along n_out; reference y = act(x @ w_dec + out_bias)."""
-    rng = np.random.default_rng(seed)
-    w = rng.normal(0, 0.02, (k_in, n_out)).astype(np.float16)
-    packed, scale, bias = group_quantize_compress_numpy(w, gs)  # [k_in, n_out / gs, gs / 4]
+    key = (n_out, k_in, gs, seed)  # (large weights take seconds to compress and decompress on the host: once per session)
+    if key not in _CASE_WEIGHTS:
+        rng = np.random.default_rng(seed)
+        w = rng.normal(0, 0.02, (k_in, n_out)).astype(np.float16)
+        packed, scale, bias = group_quantize_compress_numpy(w, gs)  # [k_in, n_out / gs, gs / 4]
+        out_bias = rng.normal(0, 1, (n_out,)).astype(np.float16)
+        w_dec = oracle.np_decompress(packed, scale, bias)  # [k_in, n_out]
+        _CASE_WEIGHTS[key] = (packed, scale, bias, out_bias, np.ascontiguousarray(w_dec.T))
+    packed, scale, bias, out_bias, w_dec_t = _CASE_WEIGHTS[key]
     x = activations(m_rows, k_in, seed + 1)
-    out_bias = rng.normal(0, 1, (n_out,)).astype(np.float16) if with_bias else None
-    w_dec = oracle.np_decompress(packed, scale, bias)  # [k_in, n_out]
-    y_ref = oracle.np_linear(x, np.ascontiguousarray(w_dec.T), out_bias, activation)
+    out_bias = out_bias if with_bias else None
+    y_ref = oracle.np_linear(x, w_dec_t, out_bias, activation)
     return x, packed, scale, bias, out_bias, y_ref
 
 
