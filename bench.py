@@ -354,7 +354,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         ms = time_launches(lambda _: graph.replay(), passes, warmup)
         results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                                        "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
-                                       "roofline": hbm_roofline("gemv_mfma_kernel / gemv_stream_single_kernel (168 launches)", w_bytes, ms)}
+                                       "roofline": hbm_roofline(("gemv_sums_kernel" if m_rows <= 2 else "gemv_stream_single_kernel / gemv_mfma_kernel" if m_rows <= 4
+                                                                else "gemv_mfma_kernel") + " (168 launches)", w_bytes, ms)}
     # (1b) the same stack with every weight in the default layout of LinearGQ (groups along the output
     # features), read from the derived copy a layer keeps after prepack_for_decode(): one launch of
     # gq_linear_knp_act_f16 per matrix replayed from a HIP graph, and the same entries as a sequence
@@ -712,7 +713,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             one_pass_two(stream_handle())
         ms = time_launches(lambda _: graph.replay(), passes, warmup)
         torch.cuda.synchronize()
-        kernel = "gemv_mfma_kernel (streaming layout; 56 launches)" if m_rows > 4 else "gemv_stream_single_kernel / gemv_mfma_kernel (streaming layout; 56 launches)"
+        kernel = ("gemv_sums_kernel" if m_rows <= 2 else "gemv_stream_single_kernel / gemv_mfma_kernel" if m_rows <= 4
+                  else "gemv_mfma_kernel") + " (streaming layout; 56 launches)"
         results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
                          "status": 0, "roofline": hbm_roofline(kernel, w_bytes, ms)}
         # the last layer's two results against single calls on the variables (and the oracle, when a test hands it over)
@@ -923,7 +925,7 @@ def main():
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
             for m in (1, 8):
                 r = bench_linear(hip, device, "gq_gemv_f16", m, n_out, k_in, 200, 20,
-                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_mfma_kernel / gemv_stream_single_kernel")
+                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_sums_kernel" if m <= 2 else "gemv_mfma_kernel")
                 extra["gemv"].append(r)
                 log(f"  gemv m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()
@@ -934,7 +936,8 @@ def main():
         for n_out, k_in in ((4096, 4096), (16384, 4096), (4096, 16384)):
             for m in (1, 8):
                 r = bench_linear(hip, device, "gq_linear_p_act_f16", m, n_out, k_in, 200, 20,
-                                 n_sets=sets_beyond_cache(n_out, k_in), kernel="gemv_mfma_kernel (streaming layout)")
+                                 n_sets=sets_beyond_cache(n_out, k_in),
+                                 kernel=("gemv_sums_kernel" if m <= 2 else "gemv_mfma_kernel") + " (streaming layout)")
                 extra["gemv_streaming_layout"].append(r)
                 log(f"  gemv, streaming layout m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
                 torch.cuda.empty_cache()

@@ -51,6 +51,11 @@ int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint1
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
                 int64_t group_size, int act, hipStream_t stream, const void *blob = nullptr);
+// One or two batch rows, group 64, k_in % 512 == 0, x / packed (or blob) 16-byte and scale / bias 4-byte aligned:
+// scale and bias applied to group sums (gq_gemv_sums.hip).  blob: NULL, or the weight's streaming-layout copy.
+int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                     const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
+                     hipStream_t stream);
 // workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
 // blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16, which the pipelined kernel then reads
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
