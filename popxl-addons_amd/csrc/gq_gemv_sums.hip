@@ -214,14 +214,20 @@ int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
                      hipStream_t stream) {
   const int64_t row_blocks = (n_out + 15) / 16;
-  // row blocks per wave as in launch_gemv: the fewest bytes per busy compute unit
+  // Row blocks per wave (1, 2 or 4; they share the x operands): the fewest bytes per busy compute unit -- the weights
+  // once, x once per workgroup (out of L2: counted half), divided by the share of the compute units' turns that the
+  // workgroups fill.  With one or two row blocks a wave takes at most 116 registers and two workgroups share a compute
+  // unit (512 places a turn), with four 178 and one (256 places, and 8 % more time for the same bytes: 16384 x 4096 at
+  // one row 8.9 us against 8.2 us with two row blocks, 28672 x 4096 15.7 against 13.8 us).
   int r = 1;
   double best = 0;
   for (int cand = 4; cand >= 1; cand >>= 1) {
-    const int64_t wgs = (row_blocks + cand - 1) / cand;
-    const double fill = (double)wgs / (double)((wgs + 255) / 256 * 256);
+    const int64_t wgs = (row_blocks + cand - 1) / cand, places = cand == 4 ? 256 : 512;
+    const double fill = wgs <= places ? (wgs < 256 ? (double)wgs / 256.0 : 1.0)
+                                      : (double)wgs / (double)((wgs + places - 1) / places * places);
     const double bytes = (double)n_out * k_in * 0.5625 + 0.5 * (double)wgs * m_rows * k_in * 2.0;
-    if (best == 0 || bytes / fill < best) best = bytes / fill, r = cand;
+    const double cost = bytes / fill * (cand == 4 ? 1.08 : 1.0);
+    if (best == 0 || cost < best) best = cost, r = cand;
   }
   const unsigned blocks = (unsigned)((row_blocks + r - 1) / r);
   const uint4_t *const weight = reinterpret_cast<const uint4_t *>(blob ? blob : packed);
