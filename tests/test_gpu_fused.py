@@ -145,6 +145,35 @@ def test_gemv_alignment_fallbacks(hip, device, oracle, gs, m_rows):
         assert normalised_error(y, y_fast.astype(np.float32)) <= REGRESSION_TOL, offsets
 
 
+@pytest.mark.parametrize("m_rows", [1, 2, 5])
+def test_gemv_outlier_activations_and_uneven_groups(hip, device, oracle, m_rows):
+    """Activations with a few values hundreds of times the rest, and weight rows whose groups differ in spread by
+    a factor of 250 and sit off zero (large biases): the kernels that apply scale and bias to group sums take the
+    codes' offsets (64 and 1024 per weight) out of sums that such activations dominate.  One and two rows run
+    that arithmetic, five rows the kernel that expands every weight; from the variables and from the copy."""
+    from popxl_addons._gq_hip import prepack_gemv
+
+    n_out, k_in = 1000, 4096
+    rng = np.random.default_rng(77)
+    spread = np.exp(rng.uniform(np.log(2e-4), np.log(5e-2), (n_out, k_in // 64, 1)))
+    centre = rng.normal(0, 0.05, (n_out, k_in // 64, 1))
+    w = (rng.normal(0, 1, (n_out, k_in // 64, 64)) * spread + centre).reshape(n_out, k_in).astype(np.float16)
+    packed, scale, bias = group_quantize_compress_numpy(w, 64)
+    w_dec = oracle.np_decompress(packed, scale, bias)
+    x = activations(m_rows, k_in, 78)
+    where = rng.choice(k_in, 12, replace=False)
+    x[:, where] = (rng.choice([-1.0, 1.0], (m_rows, 12)) * rng.uniform(100, 600, (m_rows, 12))).astype(np.float16)
+    y_ref = oracle.np_linear(x, w_dec, None)
+    assert_close(_call(hip, "gq_gemv_f16", x, packed, scale, bias, None, n_out, k_in, 64, device), y_ref, "variables")
+    dev = tuple(to_dev(a, device) for a in (packed, scale, bias))
+    copy = prepack_gemv(*dev)
+    y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    hip.call("gq_linear_p_act_f16", to_dev(x, device).data_ptr(), m_rows, 0, 0, 0, copy.blob.data_ptr(), 0, y.data_ptr(), n_out, k_in, 64,
+             0, 0, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert_close(y.cpu().numpy(), y_ref, "copy")
+
+
 @pytest.mark.parametrize("m_rows", [128, 512, 2048])
 def test_gemm_benchmark_shapes(hip, device, oracle, m_rows):
     """Benchmark configuration 4: prefill batches on the [16384 x 4096] weight."""
