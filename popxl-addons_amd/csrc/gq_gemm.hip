@@ -862,7 +862,7 @@ namespace {
 
 // The tile shape and the number of workgroups that divide K for one output tile.
 //
-// Four tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
+// Five tile shapes.  The larger the tile, the less x and weight traffic per multiply-add, but a
 // launch is as slow as its busiest compute unit: expected time = workgroups per compute unit (256 of
 // them; a last, partly filled round runs faster: fewer workgroups share memory and clocks) x time
 // per workgroup, from measured times per 1024 input features with every compute unit busy:
@@ -870,30 +870,43 @@ namespace {
 //   128 x 64   8 us    (16384 x 4096 at 128 rows: 34.5 us)
 //   256 x 128  22 us   (16384 x 4096 at 512 rows: 87 us; 16 us with an eighth of the compute units busy)
 //   256 x 256  34 us   (16384 x 4096 at 2048 rows: two rounds, 271 us; at 1024 rows one, 140 us)
+//   128 x 256  22 us   (eight waves of 128 x 32; 20.7 us for a weight in a streaming layout)
 // Fixed thresholds on the batch alone (256 x 128 from 256 rows, 256 x 256 from 1024) left weights
 // with 4096 outputs on 16 to 64 workgroups: 4096 x 4096 at 512 rows took 75.6 us, now 36 us.  With each
 // shape forced in turn, this choice was the fastest or within 2 % of it for five weight shapes
 // (16384 x 4096, 4096 x 16384, 4096 x 4096, 12288 x 4096, 8192 x 8192) at nine batches from 128 to 4096.
 //
+// 128 x 256 has the output area of 256 x 128 on twice the waves (two per SIMD hide each other's waits)
+// at twice the expansion work per multiply-add.  It wins where it wastes fewer rows (16384 x 4096 at
+// 384 rows: 192 workgroups instead of 256 with a quarter of their rows unused, 74.2 against 88.6 us,
+// from the streaming layout 62.4 against 83.7) and, on a weight in a streaming layout, whose loads
+// are whole KiB, also at the same number of workgroups (16384 x 4096 at 512 rows 76.5 against 81.5 us,
+// 12288 x 4096 61.5 against 73.3; on the three variables 87.2 against 86.6 and 73.5 against 76.0: a
+// tie goes to 256 x 128 there).  K is not divided over workgroups with this shape, so that the
+// workspace a caller sized without knowing of a streaming-layout copy serves either choice.
+//
 // With a workspace, 2 to 16 workgroups may divide the K loop of a tile (each at least four steps of
 // 64) and add their fp32 accumulators through it: priced at 4 us plus the partial sums written and
 // read at 5 TB/s.
 struct GemmPlan {
-  int shape;   // 0: 64 x 64, 1: 128 x 64, 2: 256 x 128, 3: 256 x 256
+  int shape;   // 0: 64 x 64, 1: 128 x 64, 2: 256 x 128, 3: 256 x 256, 4: 128 x 256
   int splits;  // workgroups per output tile
   int64_t tiles, tile_bytes;
   double us;   // expected time
 };
 
-GemmPlan plan_gemm(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split) {
-  static const int tile_m[4] = {64, 128, 256, 256}, tile_n[4] = {64, 64, 128, 256};
-  static const double us_per_1024[4] = {6.3, 8.0, 22.0, 34.0};
+// `streamed`: the weight is read from a streaming-layout copy.
+GemmPlan plan_gemm(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split, bool streamed) {
+  static const int tile_m[5] = {64, 128, 256, 256, 128}, tile_n[5] = {64, 64, 128, 256, 256};
+  const double us_per_1024[5] = {6.3, 8.0, 22.0, 34.0, streamed ? 20.7 : 22.0};
+  static const int order[5] = {3, 2, 4, 1, 0};  // (ties go to the earlier one)
   GemmPlan best = {1, 1, 0, 0, 1e30};
-  for (int shape = 3; shape >= 0; --shape) {  // (ties go to the larger tile)
+  for (int o = 0; o < 5; ++o) {
+    const int shape = order[o];
     if (shape == 0 && k_in % 256 != 0) continue;
     const int groups = (shape <= 1 && k_in % 256 == 0) ? 2 : 1;  // groups of waves that split K inside a workgroup
     const int64_t tiles = ((m_rows + tile_m[shape] - 1) / tile_m[shape]) * ((n_out + tile_n[shape] - 1) / tile_n[shape]);
-    for (int splits = 1; splits <= (may_split ? 16 : 1); splits *= 2) {
+    for (int splits = 1; splits <= (may_split && shape != 4 ? 16 : 1); splits *= 2) {
       const int64_t steps = k_in / 64;
       if (steps % (groups * splits) != 0 || steps / (groups * splits) < 4 || (splits > 1 && tiles > kGemmCounters)) break;
       const int64_t wgs = tiles * splits, full = wgs / 256, rest = wgs % 256;
@@ -921,7 +934,7 @@ bool gemm_pipelined_ok(const uint16_t *x, const uint16_t *packed, const uint16_t
 // What the choice above expects the pipelined kernel to take (us) -- for callers that weigh it against
 // other ways of running a batch.
 double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_split) {
-  return plan_gemm(m_rows, n_out, k_in, may_split).us;
+  return plan_gemm(m_rows, n_out, k_in, may_split, false).us;
 }
 
 // Bytes of workspace with which launch_gemm may divide K over workgroups (0: it would not): 16 KiB of
@@ -930,7 +943,7 @@ double gemm_expected_us(int64_t m_rows, int64_t n_out, int64_t k_in, bool may_sp
 int64_t gemm_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
   const bool pow2 = (group_size & (group_size - 1)) == 0;
   if (m_rows < 1 || n_out < 1 || !pow2 || group_size < 32 || k_in <= 0 || k_in % BK != 0 || (k_in / group_size) % 2 != 0) return 0;
-  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, true);
+  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, true, false);
   return plan.splits == 1 ? 0 : (int64_t)kGemmCounters * 4 + plan.splits * plan.tiles * plan.tile_bytes;
 }
 
@@ -955,8 +968,9 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
                                                                       gs_shift, act, plan.splits,                                \
                                                                       plan.splits > 1 ? workspace : nullptr, stream))
   if (gemm_pipelined_ok(x, packed, scale, bias, k_in, group_size)) {
-    const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, workspace != nullptr);
+    const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, workspace != nullptr, blob != nullptr);
     if (plan.shape == 0) return GQ_PIPE2(2, 2, 1, 1, 3, 2, 2);  // 64 x 64, two groups of 4 waves of 32 x 32
+    if (plan.shape == 4) return GQ_PIPE2(1, 8, 4, 1, 4, 1);     // 128 x 256, 8 waves of 128 x 32
     if (plan.shape == 3) return GQ_PIPE2(1, 8, 8, 1, 4, 2);     // 256 x 256, 8 waves of 256 x 32
     if (plan.shape == 2) return GQ_PIPE2(1, 4, 8, 1, 3, 1);     // 256 x 128, 4 waves of 256 x 32
     // 128 x 64 (a workgroup on every compute unit at n_out = 16384), 4 waves of 64 x 32; two such
@@ -979,10 +993,11 @@ int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 // chooses for the other layout (K is not divided over workgroups: no workspace here).
 int launch_gemm_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                     int64_t k_in, int act, hipStream_t stream) {
-  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, false);
+  const GemmPlan plan = plan_gemm(m_rows, n_out, k_in, false, true);
 #define GQ_PIPE2_KN(WM, WN, FM, FN, XS, OCC, ...) \
   launch_pipe2_kn<WM, WN, FM, FN, XS, OCC, ##__VA_ARGS__>(x, m_rows, blob, out_bias, y, n_out, k_in, act, stream)
   if (plan.shape == 0) return GQ_PIPE2_KN(2, 2, 1, 1, 3, 2, 2);
+  if (plan.shape == 4) return GQ_PIPE2_KN(1, 8, 4, 1, 4, 1);
   if (plan.shape == 3) return GQ_PIPE2_KN(1, 8, 8, 1, 4, 2);
   if (plan.shape == 2) return GQ_PIPE2_KN(1, 4, 8, 1, 3, 1);
   return GQ_PIPE2_KN(2, 2, 2, 1, 3, 1, 2);

@@ -38,9 +38,10 @@ def _run(hip, device, x, dev, blob, out_bias, n_out, k_in, act, workspace=None):
     return y.cpu().numpy()
 
 
-@pytest.mark.parametrize("m_rows", [128, 512, 2048])
+@pytest.mark.parametrize("m_rows", [128, 384, 512, 2048])
 def test_benchmark_prefill_batches(hip, device, oracle, m_rows):
-    """Benchmark configuration 4 on the derived copy: every tile shape of the pipelined kernel."""
+    """Benchmark configuration 4 on the derived copy: every tile shape of the pipelined kernel (128 x 64, 128 x 256
+    -- at 384 rows from the variables too, at 512 rows from the copy only --, 256 x 128, 256 x 256)."""
     n_out, k_in = 16384, 4096
     dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 21)
     x = activations(m_rows, k_in, 22)
