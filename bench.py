@@ -249,6 +249,18 @@ def sets_beyond_cache(n_out, k_in):
     return max(2, int(600e6 // (n_out * k_in * (0.5 + 4.0 / GROUP))) + 1)
 
 
+def one_shot_kernel_name(m_rows, n_out, k_in):
+    """The kernel that a single fused GEMV of this shape runs on (weights grouped along the input features, group 64,
+    k_in % 512 == 0, aligned operands): the library's routing, restated for the labels of the rows."""
+    if m_rows <= 2:
+        return "gemv_sums_kernel"
+    if m_rows <= 8 and k_in <= 4096 and ((n_out + 15) // 16 + 7) // 8 >= 208:
+        return "gemv_rows_kernel"
+    if m_rows <= 4 and n_out * k_in >= (72 << 20) and k_in < 8192:
+        return "gemv_stream_kernel as a sequence of one"
+    return "gemv_mfma_kernel"
+
+
 def bench_linear(hip, device, entry, m_rows, n_out, k_in, steps, warmup, n_sets, kernel):
     """One fused dequant matmul shape; weights rotated over n_sets distinct copies.  `entry` is
     gq_gemv_f16 / gq_gemm_f16 (weight [n_out, k_in], groups along k_in) or gq_linear_kn_act_f16
@@ -842,6 +854,8 @@ def main():
     ap.add_argument("--stack-modes", default="",
                     help="comma-separated schedules of the 28-layer stack to run (default: all), e.g. for a profile of one kernel")
     ap.add_argument("--stack-batches", default="1,4,8", help="batch sizes of the stack runs")
+    ap.add_argument("--gemv-shapes", default="", help="the single-launch rows after the benchmark's: these weights instead of the stack's two products (n_out x k_in, ...)")
+    ap.add_argument("--gemv-batches", default="1,4,8", help="batches of those rows")
     ap.add_argument("--knp-shapes", default="", help="--only knp: decode rows on these weights instead (n_out x k_in, e.g. 4096x20480,28672x4096)")
     ap.add_argument("--knp-batches", default="1,8", help="decode batches of the knp rows")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
@@ -940,6 +954,18 @@ def main():
                                  kernel=("gemv_sums_kernel" if m <= 2 else "gemv_mfma_kernel") + " (streaming layout)")
                 extra["gemv_streaming_layout"].append(r)
                 log(f"  gemv, streaming layout m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%})")
+                torch.cuda.empty_cache()
+    if args.only in ("gemv", "all"):
+        # the two products of a layer of the 56-entry stack schedule ([up | v | q | k] and [down | o]) as single launches, from
+        # the copy; --gemv-shapes / --gemv-batches: other weights and batches
+        shapes = [tuple(int(v) for v in s.split("x")) for s in args.gemv_shapes.split(",") if s] or [(28672, 4096), (4096, 20480)]
+        extra["gemv_stack_products"] = []
+        for n_out, k_in in shapes:
+            for m in [int(v) for v in args.gemv_batches.split(",")]:
+                r = bench_linear(hip, device, "gq_linear_p_act_f16", m, n_out, k_in, 200, 20, n_sets=sets_beyond_cache(n_out, k_in),
+                                 kernel=one_shot_kernel_name(m, n_out, k_in) + " (streaming layout)")
+                extra["gemv_stack_products"].append(r)
+                log(f"  gemv, streaming layout m={m} [{n_out}x{k_in}]: {r['us']:.1f} us, {r['weight_gbs']:.0f} GB/s weights ({r['hbm_frac']:.1%}; {r['roofline']['kernel']})")
                 torch.cuda.empty_cache()
     if args.only in ("kn", "all"):
         # the same shapes with the weight stored [k_in, n_out] and grouped along n_out: the default layout of LinearGQ

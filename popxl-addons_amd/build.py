@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libgq_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 SOURCES = ["gq_api.hip", "gq_decompress.hip", "gq_compress.hip", "gq_gemv.hip", "gq_gemv_stream.hip", "gq_gemv_flow.hip", "gq_gemm.hip", "gq_linear_kn.hip",
-           "gq_gemv_kn.hip", "gq_gemv_sums.hip"]
+           "gq_gemv_kn.hip", "gq_gemv_sums.hip", "gq_gemv_rows.hip"]
 
 # -ffp-contract=off: the decompress contract is "fp16 multiply, then fp16 add" (two roundings);
 # kernels that want an fma ask for one explicitly.  Packed-fp32 instruction selection is disabled.
@@ -34,7 +34,7 @@ NO_FMA_SOURCES = {"gq_decompress.hip": r"v_(pk_)?(fma|mad|fmac)_f16|v_fma_mix"}
 # kernels that count their outstanding vector-memory operations by hand (s_waitcnt vmcnt(N) with
 # direct-to-LDS loads): a register spill would add scratch accesses to that count
 NO_SCRATCH_SOURCES = ["gq_gemv_stream.hip", "gq_gemv_flow.hip", "gq_gemm.hip", "gq_linear_kn.hip",
-           "gq_gemv_kn.hip", "gq_gemv_sums.hip"]
+           "gq_gemv_kn.hip", "gq_gemv_sums.hip", "gq_gemv_rows.hip"]
 
 
 def _run(cmd):

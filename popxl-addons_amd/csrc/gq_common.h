@@ -56,6 +56,13 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
                      hipStream_t stream);
+// Three to eight batch rows, group 64, x / packed (or blob) / scale / bias 16-byte aligned, a shape that gemv_rows_fits
+// (k_in <= 4096, a multiple of 512; rows enough to fill the compute units): the waves of a workgroup share the rows' x
+// (gq_gemv_rows.hip).  blob: NULL, or the weight's streaming-layout copy.
+bool gemv_rows_fits(int64_t m_rows, int64_t n_out, int64_t k_in);
+int launch_gemv_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
+                     const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
+                     hipStream_t stream);
 // workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
 // blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16, which the pipelined kernel then reads
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,

@@ -275,6 +275,12 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   if (m_rows <= 2 && group_size == 64 && k_in > 0 && k_in % 512 == 0 && ((uintptr_t)x % 16) == 0 &&
       (blob || (((uintptr_t)packed % 16) == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0)))
     return launch_gemv_sums(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream);
+  // Three to eight rows on a weight whose rows alone fill the compute units (k_in <= 4096): the kernel whose waves
+  // share the rows' x
+  if (group_size == 64 && ((uintptr_t)x % 16) == 0 &&
+      (blob || (((uintptr_t)packed % 16) == 0 && ((uintptr_t)scale % 16) == 0 && ((uintptr_t)bias % 16) == 0)) &&
+      gemv_rows_fits(m_rows, n_out, k_in))
+    return launch_gemv_rows(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream);
   // Weights of 72 Mi elements or more with rows shorter than 8192 features go through the persistent
   // kernel at batches up to 4, as a sequence of one: its pipelined rings beat the one-shot kernel below
   // there (measured at one row: 20480x4096 15.1 -> 13.2 us, 24576x4096 19.7 -> 14.6 us, 32768x4096

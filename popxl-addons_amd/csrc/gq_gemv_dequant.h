@@ -36,6 +36,20 @@ __device__ __forceinline__ half8_t dequant_word(uint32_t w, half2_t s2, half2_t 
                                  __builtin_shufflevector(w2, w3, 0, 1, 2, 3), 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// 8 codes of a word as fp16 in the order (0,4,1,5,2,6,3,7) of their input features: (64 + c, 64 + c,
+// 1024 + c, 1024 + c) twice.  Plain C with the masks in vector registers the compiler cannot see
+// through (it then selects v_and_or_b32, and places the wait states a VALU write next to an MFMA needs).
+__device__ __forceinline__ half8_t sums_raw_codes(uint32_t w, uint32_t mask_lo, uint32_t mask_hi, uint32_t magic_lo,
+                                                  uint32_t magic_hi) {
+  const uint32_t hi = w >> 8;
+  uint4_t v;
+  v.x = (hi & mask_hi) | magic_hi;  // nibbles 3, 7: features 0, 4
+  v.y = (hi & mask_lo) | magic_lo;  // nibbles 2, 6: features 1, 5
+  v.z = (w & mask_hi) | magic_hi;   // nibbles 1, 5: features 2, 6
+  v.w = (w & mask_lo) | magic_lo;   // nibbles 0, 4: features 3, 7
+  return __builtin_bit_cast(half8_t, v);
+}
+
 // 8 consecutive fp16 of x -> order (0,4,1,5,2,6,3,7)
 __device__ __forceinline__ half8_t permute_x(uint4_t q) {
   uint4_t p;

@@ -30,20 +30,6 @@ constexpr int kSumsItemBytes = 4608;    // streaming layout: 4 KiB of codes, 16 
 constexpr int kSumsRegionBytes = 2560;  // per wave: 2 KiB of x (two batch rows of a chunk), 128 B of group sums, spare
 constexpr int kSumsLdsBytes = kSumsWaves * kSumsRegionBytes + 1024;  // + 1 KiB of zeros for the A rows without data
 
-// 8 codes of a word as fp16 in the order (0,4,1,5,2,6,3,7) of their input features: (64 + c, 64 + c,
-// 1024 + c, 1024 + c) twice.  Plain C with the masks in vector registers the compiler cannot see
-// through (it then selects v_and_or_b32, and places the wait states a VALU write next to an MFMA needs).
-__device__ __forceinline__ half8_t sums_raw_codes(uint32_t w, uint32_t mask_lo, uint32_t mask_hi, uint32_t magic_lo,
-                                                  uint32_t magic_hi) {
-  const uint32_t hi = w >> 8;
-  uint4_t v;
-  v.x = (hi & mask_hi) | magic_hi;  // nibbles 3, 7: features 0, 4
-  v.y = (hi & mask_lo) | magic_lo;  // nibbles 2, 6: features 1, 5
-  v.z = (w & mask_hi) | magic_hi;   // nibbles 1, 5: features 2, 6
-  v.w = (w & mask_lo) | magic_lo;   // nibbles 0, 4: features 3, 7
-  return __builtin_bit_cast(half8_t, v);
-}
-
 // XM: 1 or 2 >= m_rows.
 template <int R, int XM, bool BLOB>
 __global__ __launch_bounds__(kSumsWaves * 64) void gemv_sums_kernel(const half_t *__restrict__ x, int m_rows,

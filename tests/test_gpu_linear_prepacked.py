@@ -54,16 +54,36 @@ def test_benchmark_prefill_batches(hip, device, oracle, m_rows):
 @pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (16384, 4096), (4096, 16384), (28672, 4096), (1000, 1536), (16, 512)])
 @pytest.mark.parametrize("m_rows", [1, 3, 4, 8, 16])
 def test_decode_batches(hip, device, oracle, n_out, k_in, m_rows):
-    """Up to 16 rows the one-shot GEMV kernel reads the copy (every load 1 KiB contiguous, read once) -- on the
-    widest weight at up to 4 rows the persistent kernel as a sequence of one: the oracle's result, and the bits
-    of the same call on the variables where the same kernel runs."""
+    """Up to 16 rows the GEMV kernels read the copy (every load 1 KiB contiguous, read once): the oracle's result,
+    and the bits of the same call on the variables (the same kernel runs on either)."""
     dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 41)
     x = activations(m_rows, k_in, 42 + m_rows)
     ob = np.random.default_rng(43).normal(0, 1, (n_out,)).astype(np.float16) if m_rows % 2 else None
     y = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 1)
     assert_close(y, oracle.np_linear(x, w_dec, ob, "relu"), (n_out, k_in, m_rows))
-    if not (n_out == 28672 and m_rows <= 4):
-        assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 1), "against the variables")
+    assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, 1), "against the variables")
+
+
+@pytest.mark.parametrize("n_out,k_in", [(28672, 4096), (28712, 1024), (32768, 512), (3400, 1536)])
+@pytest.mark.parametrize("m_rows", [3, 4, 5, 6, 7, 8])
+def test_three_to_eight_rows_on_wide_weights(hip, device, oracle, n_out, k_in, m_rows):
+    """Weights whose rows alone fill the compute units, k_in <= 4096: the kernel whose waves share the batch rows'
+    x (4 x 4 or 2 x 8 (group, batch row) combinations per accumulator; batch rows that do not fill them; a last
+    group of row blocks with waves that have no rows, a last row block with 8 rows).  3400 x 1536 stays with
+    the other kernels.  The oracle's result from the copy and from the variables, the same bits from both."""
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 41 if n_out == 28672 else 61)
+    x = activations(m_rows, k_in, 62 + m_rows)
+    ob = np.random.default_rng(63).normal(0, 1, (n_out,)).astype(np.float16) if m_rows % 2 else None
+    act, name = ((2, "gelu_tanh") if m_rows == 6 else (0, None))
+    y = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, act)
+    assert_close(y, oracle.np_linear(x, w_dec, ob, name), (n_out, k_in, m_rows))
+    assert_bits_equal(y, _run(hip, device, x, dev, None, ob, n_out, k_in, act), "against the variables")
+    only_copy = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+    xd, od = to_dev(x, device), None if ob is None else to_dev(ob, device)
+    hip.call("gq_linear_p_act_f16", xd.data_ptr(), m_rows, 0, 0, 0, copy.blob.data_ptr(), 0 if od is None else od.data_ptr(),
+             only_copy.data_ptr(), n_out, k_in, 64, act, 0, 0, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert_bits_equal(only_copy.cpu().numpy(), y, "the copy alone")
 
 
 @pytest.mark.parametrize("n_out,k_in,m_rows", [(4096, 4096, 300), (4096, 16384, 128), (4104, 512, 300), (8200, 1024, 777),
