@@ -366,8 +366,7 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         ms = time_launches(lambda _: graph.replay(), passes, warmup)
         results["per_launch_graph"] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6,
                                        "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
-                                       "roofline": hbm_roofline(("gemv_sums_kernel" if m_rows <= 2 else "gemv_stream_single_kernel / gemv_mfma_kernel" if m_rows <= 4
-                                                                else "gemv_mfma_kernel") + " (168 launches)", w_bytes, ms)}
+                                       "roofline": hbm_roofline(one_shot_kernel_name(m_rows, ffn, hidden) + " (168 launches)", w_bytes, ms)}
     # (1b) the same stack with every weight in the default layout of LinearGQ (groups along the output
     # features), read from the derived copy a layer keeps after prepack_for_decode(): one launch of
     # gq_linear_knp_act_f16 per matrix replayed from a HIP graph, and the same entries as a sequence
@@ -725,8 +724,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             one_pass_two(stream_handle())
         ms = time_launches(lambda _: graph.replay(), passes, warmup)
         torch.cuda.synchronize()
-        kernel = ("gemv_sums_kernel" if m_rows <= 2 else "gemv_stream_single_kernel / gemv_mfma_kernel" if m_rows <= 4
-                  else "gemv_mfma_kernel") + " (streaming layout; 56 launches)"
+        names = [one_shot_kernel_name(m_rows, ffn + 3 * hidden, hidden), one_shot_kernel_name(m_rows, hidden, ffn + hidden)]
+        kernel = " / ".join(dict.fromkeys(names)) + " (streaming layout; 56 launches)"
         results[mode] = {"us_per_pass": ms * 1e3, "weight_gbs": w_bytes / ms / 1e6, "hbm_frac": w_bytes / ms / 1e6 / HBM_PEAK_GBS,
                          "status": 0, "roofline": hbm_roofline(kernel, w_bytes, ms)}
         # the last layer's two results against single calls on the variables (and the oracle, when a test hands it over)
