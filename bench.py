@@ -699,21 +699,18 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         torch.cuda.synchronize()
         wide = torch.empty((m_rows, ffn + 3 * hidden), dtype=torch.float16, device=device)
         h_out = [torch.empty((m_rows, hidden), dtype=torch.float16, device=device) for _ in range(2)]
-        # (more than one row: x of the joint product is gathered by a copy, which stands for the attention and
-        # activation kernels that a model has between the two launches anyway)
-        joint_x = wide if m_rows == 1 else torch.empty((m_rows, ffn + hidden), dtype=torch.float16, device=device)
+        # (x of the joint product is the first ffn + hidden columns of `wide`, read where they lie: rows a stride apart)
+        joint_x = wide[:, : ffn + hidden]
 
         def layer_entry(stream, x, copy, y):
-            hip.call("gq_linear_p_act_f16", x.data_ptr(), m_rows, 0, 0, 0, copy.blob.data_ptr(), 0, y.data_ptr(), copy.n_out, copy.k_in,
-                     GROUP, 0, 0, 0, stream)
+            hip.call("gq_linear_p_strided_f16", x.data_ptr(), x.stride(0), m_rows, 0, 0, 0, copy.blob.data_ptr(), 0, y.data_ptr(),
+                     copy.n_out, copy.k_in, GROUP, 0, stream)
 
         def one_pass_two(stream):
             h = h0_joint
             for layer in range(n_layers):
                 _, first_copy, _, out_copy = two[layer]
                 layer_entry(stream, h, first_copy, wide)
-                if m_rows > 1:
-                    joint_x.copy_(wide[:, : ffn + hidden])
                 h = h_out[layer % 2]
                 layer_entry(stream, joint_x, out_copy, h)
 
@@ -732,8 +729,8 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
         worst, worst_oracle = 0.0, 0.0
         h_last = h_out[(n_layers - 2) % 2]
         first, _, out, _ = two[n_layers - 1]
-        # (at one row joint_x IS the wide result: the product's x is its first ffn + hidden values, not all of them)
-        for x_in, (p, s_, b), y in ((h_last, first, wide), (joint_x[:, : ffn + hidden], out, h_out[(n_layers - 1) % 2])):
+        # (the single calls read a gathered copy of the joint product's x)
+        for x_in, (p, s_, b), y in ((h_last, first, wide), (joint_x.contiguous(), out, h_out[(n_layers - 1) % 2])):
             assert x_in.is_contiguous() and x_in.shape[1] * 2 == p.shape[1] * p.shape[2] * 8 and y.shape[1] == p.shape[0]
             ref = torch.empty_like(y)
             hip.call("gq_gemv_f16", x_in.data_ptr(), m_rows, p.data_ptr(), s_.data_ptr(), b.data_ptr(), 0, ref.data_ptr(),

@@ -170,6 +170,21 @@ int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packe
                         int64_t workspace_bytes, void *stream);
 
 /*
+ * gq_linear_p_act_f16 at decode batches (m_rows <= 16) for an x whose rows are `x_row_stride` elements
+ * apart (>= k_in): a column slice of a wider matrix -- e.g. the part of the output of fused projections
+ * (LinearGQ.fuse) that the next layer consumes -- without a copy that gathers it.  No counterpart in the
+ * reference (a popxl slice is a view of the static graph, popxl_addons/layers/linear_gq.py:99-109 sees a
+ * tensor).  The same kernels and results as the call on a gathered x; x_row_stride == k_in is that call.
+ * The fast kernels need every row of x 16-byte aligned (x and x_row_stride % 8 == 0; with packed, scale and
+ * bias NULL anything else is GQ_ERR_MISALIGNED).  m_rows > 16: GQ_ERR_UNSUPPORTED (gather x, or call per 16
+ * rows); x_row_stride < k_in: GQ_ERR_BAD_SHAPE.  blob may be NULL (the three variables are read).
+ */
+int gq_linear_p_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m_rows, const uint16_t *packed,
+                            const uint16_t *scale, const uint16_t *bias, const void *blob, const uint16_t *out_bias,
+                            uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation,
+                            void *stream);
+
+/*
  * Fused decompress + matmul, groups along the OUTPUT features: the computation of LinearGQ.build
  * with dim = -1 or 1, the constructor default (popxl_addons/layers/linear_gq.py:26, 59-62, 99-109):
  *   w = decompress(packed, scale, bias)      [k_in, n_out]

@@ -201,6 +201,36 @@ int gq_linear_p_act_f16(const uint16_t *x, int64_t m_rows, const uint16_t *packe
                          (hipStream_t)stream, blob);
 }
 
+int gq_linear_p_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m_rows, const uint16_t *packed,
+                            const uint16_t *scale, const uint16_t *bias, const void *blob, const uint16_t *out_bias,
+                            uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation,
+                            void *stream) {
+  const bool only_blob = blob && !packed && !scale && !bias;
+  const uint16_t *const stand_in = static_cast<const uint16_t *>(blob);
+  const int rc = gq::check_linear_args("gq_linear_p_strided_f16", x, m_rows, only_blob ? stand_in : packed,
+                                       only_blob ? stand_in : scale, only_blob ? stand_in : bias, out_bias, y, n_out, k_in,
+                                       group_size);
+  if (rc <= 0) return rc;
+  if (x_row_stride < k_in)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_p_strided_f16: x_row_stride=%lld is less than k_in=%lld", (long long)x_row_stride,
+                    (long long)k_in);
+  if (m_rows > 16)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_p_strided_f16: m_rows=%lld; rows of x apart are taken up to 16 rows "
+                    "(gather x, or call per 16 rows)", (long long)m_rows);
+  if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_p_strided_f16: unknown activation %d", (int)activation);
+  if (blob) {
+    const int64_t blob_bytes = gq_gemv_prepacked_bytes(n_out, k_in, group_size);
+    if (blob_bytes < 0) return (int)blob_bytes;  // (no streaming layout for this shape: the message is set)
+    if (gq::misaligned(blob, 16)) return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_p_strided_f16: blob must be 16-byte aligned");
+    if (only_blob && (gq::misaligned(x, 16) || x_row_stride % 8 != 0))
+      return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_p_strided_f16: without packed, scale and bias, every row of x must be "
+                      "16-byte aligned (x, and x_row_stride %% 8 == 0)");
+  }
+  return gq::launch_gemv(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, (int)activation, (hipStream_t)stream,
+                         blob, x_row_stride);
+}
+
 int64_t gq_linear_kn_workspace_bytes(int64_t m_rows, int64_t n_out, int64_t k_in, int64_t group_size) {
   if (m_rows < 0 || n_out < 0 || k_in < 0 || group_size <= 0)
     return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_kn_workspace_bytes: negative size");

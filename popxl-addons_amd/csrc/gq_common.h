@@ -48,21 +48,22 @@ __device__ __forceinline__ float apply_activation(float v, int act) {
 int launch_decompress(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, uint16_t *out,
                       int64_t rows, int64_t n_groups, int64_t n_ids, bool transposed, hipStream_t stream);
 // blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16 (packed, scale, bias may then be NULL)
+// ldx: elements from a row of x to the next (0: k_in) -- here and in the two launchers below
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream, const void *blob = nullptr);
+                int64_t group_size, int act, hipStream_t stream, const void *blob = nullptr, int64_t ldx = 0);
 // One or two batch rows, group 64, k_in % 512 == 0, x / packed (or blob) 16-byte and scale / bias 4-byte aligned:
 // scale and bias applied to group sums (gq_gemv_sums.hip).  blob: NULL, or the weight's streaming-layout copy.
 int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
-                     hipStream_t stream);
+                     hipStream_t stream, int64_t ldx = 0);
 // Three to eight batch rows, group 64, x / packed (or blob) / scale / bias 16-byte aligned, a shape that gemv_rows_fits
 // (k_in <= 4096, a multiple of 512; rows enough to fill the compute units): the waves of a workgroup share the rows' x
 // (gq_gemv_rows.hip).  blob: NULL, or the weight's streaming-layout copy.
 bool gemv_rows_fits(int64_t m_rows, int64_t n_out, int64_t k_in);
 int launch_gemv_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
-                     hipStream_t stream);
+                     hipStream_t stream, int64_t ldx = 0);
 // workspace: NULL, or gemm_workspace_bytes() bytes (first 16 KiB zero), with which K may be divided over workgroups
 // blob: NULL, or the same weight in the streaming layout of gq_gemv_prepack_f16, which the pipelined kernel then reads
 int launch_gemm(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,

@@ -48,7 +48,7 @@ template <int NWAVES, int R, int GS, bool FULL, int XM, bool BLOB = false>
 __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
     const half_t *__restrict__ x, int m_rows, const uint4_t *__restrict__ packed, const half_t *__restrict__ scale,
     const half_t *__restrict__ bias, const half_t *__restrict__ out_bias, half_t *__restrict__ y, int n_out, int k_in,
-    int gs_shift, int act) {
+    int gs_shift, int act, int ldx) {
   // per wave: the x chunk of up to XM batch rows while the wave walks K, its partial sums at the end
   constexpr int kRegion = gemv_region_bytes(R, XM);
   extern __shared__ __attribute__((aligned(16))) char region_base[];
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemv_mfma_kernel(
       for (int m = 0; m < XM; ++m) {
         xq[m] = uint4_t{0u, 0u, 0u, 0u};
         if (m < m_rows && (FULL || c * 512 + lane * 8 < k_in))  // (k_in is a multiple of 128: a piece is whole or absent)
-          xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * k_in + c * 512 + lane * 8);
+          xq[m] = *reinterpret_cast<const uint4_t *>(x + (int64_t)m * ldx + c * 512 + lane * 8);  // (rows of x: ldx elements apart)
       }
     }
     uint4_t wq[R][4];
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
                                                            const half_t *__restrict__ scale,
                                                            const half_t *__restrict__ bias,
                                                            const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                           int n_out, int k_in, int group_size, int act) {
+                                                           int n_out, int k_in, int group_size, int act, int ldx) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= n_out) return;
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
     for (int m = 0; m < 16; ++m)
       if (m < m_rows) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[m] += (float)x[(int64_t)m * k_in + wi * 4 + j] * wv[j];
+        for (int j = 0; j < 4; ++j) acc[m] += (float)x[(int64_t)m * ldx + wi * 4 + j] * wv[j];
       }
   }
 #pragma unroll
@@ -263,8 +263,10 @@ __global__ __launch_bounds__(256) void gemv_generic_kernel(const half_t *__restr
 // k_in % 512 == 0); with x and the blob 16-byte aligned the kernels read it and packed, scale, bias may be NULL.
 int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale,
                 const uint16_t *bias, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in,
-                int64_t group_size, int act, hipStream_t stream, const void *blob) {
-  if (blob && (group_size != 64 || k_in % 512 != 0 || k_in <= 0 || ((uintptr_t)x % 16) != 0 || ((uintptr_t)blob % 16) != 0)) {
+                int64_t group_size, int act, hipStream_t stream, const void *blob, int64_t ldx) {
+  if (ldx == 0) ldx = k_in;  // rows of x: ldx elements apart (a multiple of 8 where x must be 16-byte aligned)
+  const bool x_aligned = ((uintptr_t)x % 16) == 0 && ldx % 8 == 0;  // every row of x on a 16-byte boundary
+  if (blob && (group_size != 64 || k_in % 512 != 0 || k_in <= 0 || !x_aligned || ((uintptr_t)blob % 16) != 0)) {
     if (!packed || !scale || !bias)
       return fail(GQ_ERR_UNSUPPORTED, "a weight in the streaming layout needs group_size 64, k_in %% 512 == 0 and 16-byte aligned x");
     blob = nullptr;  // (the variables serve)
@@ -272,15 +274,15 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   // One or two batch rows on group 64 and whole chunks: the kernel that applies scale and bias to group sums
   // (five vector instructions per eight weights instead of thirteen; on the large weights of the next rule it
   // measured 14.1 / 11.1 / 11.9 us at one row on 28672 / 20480 / 24576 x 4096 against 15.4 / 12.6 / 14.2 us).
-  if (m_rows <= 2 && group_size == 64 && k_in > 0 && k_in % 512 == 0 && ((uintptr_t)x % 16) == 0 &&
+  if (m_rows <= 2 && group_size == 64 && k_in > 0 && k_in % 512 == 0 && x_aligned &&
       (blob || (((uintptr_t)packed % 16) == 0 && ((uintptr_t)scale % 4) == 0 && ((uintptr_t)bias % 4) == 0)))
-    return launch_gemv_sums(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream);
+    return launch_gemv_sums(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream, ldx);
   // Three to eight rows on a weight whose rows alone fill the compute units (k_in <= 4096): the kernel whose waves
   // share the rows' x
-  if (group_size == 64 && ((uintptr_t)x % 16) == 0 &&
+  if (group_size == 64 && x_aligned &&
       (blob || (((uintptr_t)packed % 16) == 0 && ((uintptr_t)scale % 16) == 0 && ((uintptr_t)bias % 16) == 0)) &&
       gemv_rows_fits(m_rows, n_out, k_in))
-    return launch_gemv_rows(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream);
+    return launch_gemv_rows(x, m_rows, packed, scale, bias, blob, out_bias, y, n_out, k_in, act, stream, ldx);
   // Weights of 72 Mi elements or more with rows shorter than 8192 features go through the persistent
   // kernel at batches up to 4, as a sequence of one: its pipelined rings beat the one-shot kernel below
   // there (measured at one row: 20480x4096 15.1 -> 13.2 us, 24576x4096 19.7 -> 14.6 us, 32768x4096
@@ -288,7 +290,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   // 11.6 against 12.9 us).  With longer rows a wave of the one-shot kernel has several chunks to
   // overlap and wins (4096x16384 at one row: 12.0 against 14.5 us; 8192x8192: 13.3 against 14.1).
   const bool large = n_out * k_in >= ((int64_t)72 << 20) && k_in < 8192;
-  if (large && m_rows <= 4) {
+  if (large && m_rows <= 4 && ldx == k_in) {  // (a sequence entry's x is contiguous)
     const int rc = blob ? launch_gemv_streamed(x, m_rows, static_cast<const uint16_t *>(blob), nullptr, nullptr, out_bias, y, n_out,
                                                k_in, group_size, act, stream)
                         : launch_gemv_streamed(x, m_rows, packed, scale, bias, out_bias, y, n_out, k_in, group_size, act, stream);
@@ -299,7 +301,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
     scale = bias = nullptr;
   }
   const bool pow2 = (group_size & (group_size - 1)) == 0;
-  const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && ((uintptr_t)x % 16) == 0 &&
+  const bool fast_ok = pow2 && group_size >= 32 && k_in % 128 == 0 && k_in > 0 && x_aligned &&
                        ((uintptr_t)packed % 16) == 0;
   if (fast_ok) {
     const int gs_shift = __builtin_ctzll((unsigned long long)group_size);
@@ -332,7 +334,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
 #define GQ_GEMV_ARGS                                                                                      \
   reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const uint4_t *>(packed),            \
       reinterpret_cast<const half_t *>(scale), reinterpret_cast<const half_t *>(bias),                    \
-      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act
+      reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, gs_shift, act, (int)ldx
 #define GQ_GEMV_LAUNCH(NW, R, GS, FULL, XM, BLOB)                                                            \
   do {                                                                                                    \
     constexpr int lds_bytes = NW * gemv_region_bytes(R, XM);                                              \
@@ -384,7 +386,7 @@ int launch_gemv(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const
   gemv_generic_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(
       reinterpret_cast<const half_t *>(x), (int)m_rows, packed, reinterpret_cast<const half_t *>(scale),
       reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias),
-      reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, (int)group_size, act);
+      reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, (int)group_size, act, (int)ldx);
   return check_launch("gemv_generic_kernel");
 }
 
@@ -426,7 +428,7 @@ int launch_gemv_generic_rows(const uint16_t *x, int64_t m_rows, const uint16_t *
     gemv_generic_kernel<<<dim3(blocks), dim3(256), 0, stream>>>(
         reinterpret_cast<const half_t *>(x) + m0 * k_in, m, packed, reinterpret_cast<const half_t *>(scale),
         reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias),
-        reinterpret_cast<half_t *>(y) + m0 * n_out, (int)n_out, (int)k_in, (int)group_size, act);
+        reinterpret_cast<half_t *>(y) + m0 * n_out, (int)n_out, (int)k_in, (int)group_size, act, (int)k_in);
   }
   return check_launch("gemv_generic_kernel");
 }

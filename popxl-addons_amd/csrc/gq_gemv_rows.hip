@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kRowsWaves * 64) void gemv_rows_kernel(const half_t
                                                                    const half_t *__restrict__ scale,
                                                                    const half_t *__restrict__ bias,
                                                                    const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                                   int n_out, int k_in, int act) {
+                                                                   int n_out, int k_in, int act, int ldx) {
   static_assert(XM == 4 || XM == 8, "batch rows of an accumulator");
   constexpr int MB = XM;      // batch rows of an accumulator (16 / MB groups)
   constexpr int NA = MB / 2;  // accumulators per chunk
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kRowsWaves * 64) void gemv_rows_kernel(const half_t
     for (int p = wave; p < n_chunks * XM; p += kRowsWaves) {
       const int cl = p / XM, m = p % XM;
       const uint4_t xq = *reinterpret_cast<const uint4_t *>(reinterpret_cast<const char *>(x) + lane * 16 +
-                                                            ((int64_t)min(m, m_rows - 1) * k_in + cl * 512) * 2);
+                                                            ((int64_t)min(m, m_rows - 1) * ldx + cl * 512) * 2);  // (rows of x: ldx elements apart)
       float sx = 0.f, sw = 0.f;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -227,7 +227,7 @@ bool gemv_rows_fits(int64_t m_rows, int64_t n_out, int64_t k_in) {
 // streaming-layout copy.
 int launch_gemv_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
-                     hipStream_t stream) {
+                     hipStream_t stream, int64_t ldx) {
   const int xm = m_rows <= 4 ? 4 : 8;
   const unsigned groups = (unsigned)(((n_out + 15) / 16 + kRowsWaves - 1) / kRowsWaves);
   const uint4_t *const weight = reinterpret_cast<const uint4_t *>(blob ? blob : packed);
@@ -251,7 +251,7 @@ int launch_gemv_rows(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
     gemv_rows_kernel<1, XM, BLOB><<<dim3(groups), dim3(kRowsWaves * 64), lds_bytes, stream>>>(                        \
         reinterpret_cast<const half_t *>(x), (int)m_rows, weight, reinterpret_cast<const half_t *>(scale),            \
         reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias),                           \
-        reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, act);                                                   \
+        reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, act, (int)(ldx ? ldx : k_in));                          \
   } while (0)
   if (blob && xm == 4) GQ_ROWS_LAUNCH(4, true);
   else if (blob) GQ_ROWS_LAUNCH(8, true);

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kSumsWaves * 64) void gemv_sums_kernel(const half_t
                                                                    const half_t *__restrict__ scale,
                                                                    const half_t *__restrict__ bias,
                                                                    const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                                   int n_out, int k_in, int act) {
+                                                                   int n_out, int k_in, int act, int ldx) {
   extern __shared__ __attribute__((aligned(16))) char sums_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kc = lane >> 4;
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kSumsWaves * 64) void gemv_sums_kernel(const half_t
     uint32_t sdw[R], bdw[R];
 #pragma unroll
     for (int m = 0; m < XM; ++m)
-      xq[m] = *reinterpret_cast<const uint4_t *>(x_lane + ((int64_t)min(m, m_rows - 1) * k_in + c * 512) * 2);
+      xq[m] = *reinterpret_cast<const uint4_t *>(x_lane + ((int64_t)min(m, m_rows - 1) * ldx + c * 512) * 2);  // (rows of x: ldx elements apart)
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       sdw[i] = *(srow[i] + (BLOB ? c * (kSumsItemBytes / 4) : c * 4));
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kSumsWaves * 64) void gemv_sums_kernel(const half_t
 // `blob`: NULL (the three variables are read) or the weight's streaming-layout copy.
 int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, const uint16_t *scale, const uint16_t *bias,
                      const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int act,
-                     hipStream_t stream) {
+                     hipStream_t stream, int64_t ldx) {
   const int64_t row_blocks = (n_out + 15) / 16;
   // Row blocks per wave (1, 2 or 4; they share the x operands): the fewest bytes per busy compute unit -- the weights
   // once, x once per workgroup (out of L2: counted half), divided by the share of the compute units' turns that the
@@ -221,7 +221,7 @@ int launch_gemv_sums(const uint16_t *x, int64_t m_rows, const uint16_t *packed, 
   gemv_sums_kernel<R, XM, BLOB><<<dim3(blocks), dim3(kSumsWaves * 64), kSumsLdsBytes, stream>>>(                      \
       reinterpret_cast<const half_t *>(x), (int)m_rows, weight, reinterpret_cast<const half_t *>(scale),              \
       reinterpret_cast<const half_t *>(bias), reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), \
-      (int)n_out, (int)k_in, act)
+      (int)n_out, (int)k_in, act, (int)(ldx ? ldx : k_in))
 #define GQ_SUMS_BY_R(XM, BLOB)                   \
   do {                                           \
     if (r == 4) GQ_SUMS_LAUNCH(4, XM, BLOB);     \

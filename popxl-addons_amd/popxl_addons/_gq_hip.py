@@ -43,6 +43,7 @@ EXPORTS = (
     "gq_gemm_workspace_bytes",
     "gq_linear_act_ws_f16",
     "gq_linear_p_act_f16",
+    "gq_linear_p_strided_f16",
     "gq_linear_kn_workspace_bytes",
     "gq_linear_kn_act_f16",
     "gq_linear_kn_act_noalloc_f16",
@@ -108,6 +109,8 @@ def load():
     lib.gq_linear_act_ws_f16.restype = ctypes.c_int
     lib.gq_linear_p_act_f16.argtypes = [p, i64, p, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]
     lib.gq_linear_p_act_f16.restype = ctypes.c_int
+    lib.gq_linear_p_strided_f16.argtypes = [p, i64, i64, p, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p]
+    lib.gq_linear_p_strided_f16.restype = ctypes.c_int
     lib.gq_linear_kn_workspace_bytes.argtypes = [i64, i64, i64, i64]
     lib.gq_linear_kn_workspace_bytes.restype = i64
     lib.gq_linear_kn_act_f16.argtypes = [p, i64, p, p, p, p, p, i64, i64, i64, ctypes.c_int32, p, i64, p]

@@ -126,7 +126,14 @@ class LinearGQ:
             raise ValueError(f"LinearGQ: x has {in_features} features but weight_compressed is {v.weight_compressed.shape}")
         b = v.bias.data if self.bias else None
 
-        x2 = x.reshape(-1, in_features).contiguous()
+        # A decode batch that is a column slice of a wider matrix (part of the output of fused projections, say)
+        # is read where it lies, its rows a stride apart; anything else is gathered into a contiguous x.
+        x_row_stride = 0
+        if (self.dim == 0 and x.dim() == 2 and not x.is_contiguous() and x.stride(1) == 1 and x.stride(0) >= in_features
+                and 0 < x.shape[0] <= 16):
+            x2, x_row_stride = x, x.stride(0)
+        else:
+            x2 = x.reshape(-1, in_features).contiguous()
         m_rows = x2.shape[0]
         with torch.cuda.device(x.device):
             y = torch.empty((m_rows, self.out_features), dtype=torch.float16, device=x.device)
@@ -144,7 +151,10 @@ class LinearGQ:
                 act,
             )
             stream = torch.cuda.current_stream(x.device).cuda_stream
-            if self.dim == 0:
+            if x_row_stride:
+                blob = 0 if self._decode_copy is None else self._decode_copy.blob.data_ptr()
+                _gq_hip.call("gq_linear_p_strided_f16", args[0], x_row_stride, *args[1:5], blob, *args[5:], stream)
+            elif self.dim == 0:
                 # (few output tiles: several workgroups divide the input features of a tile through a workspace)
                 need = _gq_hip.load().gq_gemm_workspace_bytes(m_rows, self.out_features, in_features, self.group_size)
                 ws = _gq_hip.linear_kn_workspace(x.device, need) if need > 0 else None

@@ -128,6 +128,67 @@ def test_the_copy_alone(hip, device, oracle, n_out, k_in, m_rows):
         assert_bits_equal(y.cpu().numpy(), _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 0, workspace), "with the variables")
 
 
+@pytest.mark.parametrize("n_out,k_in", [(4096, 4096), (28672, 4096), (4096, 16384), (1000, 1536)])
+@pytest.mark.parametrize("m_rows", [1, 2, 4, 8, 16])
+def test_rows_of_x_a_stride_apart(hip, device, oracle, n_out, k_in, m_rows):
+    """gq_linear_p_strided_f16: x as a column slice of a wider matrix (rows 16-byte aligned: every kernel of the
+    decode batches reads it where it lies) gives the bits of the call on the gathered x, from the copy, from the
+    variables and from the copy alone; a slice whose rows are NOT 16-byte aligned runs the kernels for a
+    misaligned x on the variables (the oracle's result)."""
+    dev, copy, w_dec = _weight(hip, device, oracle, n_out, k_in, 41 if n_out in (28672, 1000) or k_in == 16384 else 31)
+    wide = activations(m_rows, k_in + 200, 72 + m_rows)
+    wd = to_dev(wide, device)
+    ob = np.random.default_rng(73).normal(0, 1, (n_out,)).astype(np.float16)
+    od = to_dev(ob, device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def strided(offset, variables, blob):
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        v = [t.data_ptr() for t in dev] if variables else [0, 0, 0]
+        hip.call("gq_linear_p_strided_f16", wd.data_ptr() + 2 * offset, k_in + 200, m_rows, *v, copy.blob.data_ptr() if blob else 0,
+                 od.data_ptr(), y.data_ptr(), n_out, k_in, 64, 1, stream)
+        torch.cuda.synchronize()
+        return y.cpu().numpy()
+
+    for offset in (0, 136):
+        x = np.ascontiguousarray(wide[:, offset : offset + k_in])
+        gathered = _run(hip, device, x, dev, copy.blob, ob, n_out, k_in, 1)
+        assert_close(gathered, oracle.np_linear(x, w_dec, ob, "relu"), (n_out, k_in, m_rows, offset))
+        for variables, blob in ((True, True), (True, False), (False, True)):
+            assert_bits_equal(strided(offset, variables, blob), gathered, (offset, variables, blob))
+    x = np.ascontiguousarray(wide[:, 3 : 3 + k_in])
+    assert_close(strided(3, True, True), oracle.np_linear(x, w_dec, ob, "relu"), "rows of x not 16-byte aligned")
+    with pytest.raises(GQHipError) as e:
+        strided(3, False, True)
+    assert e.value.code == GQ_ERR_MISALIGNED
+
+
+def test_layer_reads_a_column_slice_where_it_lies(hip, device, oracle):
+    """LinearGQ(dim=0).build on a decode batch that is a column slice of a wider matrix: no gather, the result of the
+    gathered call bit for bit; a slice of more than 16 rows is gathered as before."""
+    from popxl_addons.layers.linear_gq import LinearGQ
+
+    n_out, k_in = 4096, 4096
+    layer = LinearGQ(n_out, bias=False, group_size=64, dim=0)
+    layer.init_variables(k_in, torch.float16, device)
+    (p, s, b), _, w_dec = _weight(hip, device, oracle, n_out, k_in, 31)
+    v = layer.variables
+    v.weight_compressed.data.copy_(p.reshape(v.weight_compressed.shape))
+    v.weight_decompression_scale.data.copy_(s.reshape(v.weight_decompression_scale.shape))
+    v.weight_decompression_bias.data.copy_(b.reshape(v.weight_decompression_bias.shape))
+    for with_copy in (False, True):
+        if with_copy:
+            layer.prepack_for_decode()
+        for m_rows in (4, 40):
+            wide = to_dev(activations(m_rows, k_in + 512, 80 + m_rows), device)
+            part = wide[:, 256 : 256 + k_in]
+            assert not part.is_contiguous()
+            y = layer(part).cpu().numpy()
+            assert_bits_equal(y, layer(part.contiguous()).cpu().numpy(), (with_copy, m_rows))
+            assert_close(y, oracle.np_linear(part.cpu().numpy(), w_dec, None), (with_copy, m_rows))
+    layer._decode_copy = None
+
+
 def test_without_the_copy_it_is_the_workspace_entry_point(hip, device, oracle):
     n_out, k_in, m_rows = 4096, 4096, 256
     dev, _, _ = _weight(hip, device, oracle, n_out, k_in, 31)
