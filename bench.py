@@ -433,20 +433,16 @@ def bench_stack(hip, device, m_rows, passes, warmup, n_layers=28, hidden=4096, f
             h_in = (torch.randn((m_rows, hidden), generator=g, device=device, dtype=torch.float32) * 0.1).to(torch.float16)
             wide = torch.empty((m_rows, ffn + 3 * hidden), dtype=torch.float16, device=device)
             h_out = [torch.empty((m_rows, hidden), dtype=torch.float16, device=device) for _ in range(2)]
-            # (at one batch row x of the joint product is the first ffn + hidden values of the wide result;
-            # with more rows it is gathered by a copy, which stands for the attention and activation kernels
-            # that a model has between the two anyway)
-            joint_x = wide if m_rows == 1 else torch.empty((m_rows, ffn + hidden), dtype=torch.float16, device=device)
+            # (x of the joint product is the first ffn + hidden columns of the wide result, read where they lie: rows a
+            # stride apart)
 
             def one_pass_two(stream):
                 h = h_in
                 for layer in range(n_layers):
                     knp(stream, h, first_w[layer], wide)
-                    if m_rows > 1:
-                        joint_x.copy_(wide[:, : ffn + hidden])
                     h = h_out[layer % 2]
-                    hip.call("gq_linear_knp_act_f16", joint_x.data_ptr(), m_rows, out_w[layer].blob.data_ptr(), 0, h.data_ptr(), hidden,
-                             ffn + hidden, GROUP, 0, stream)
+                    hip.call("gq_linear_knp_strided_f16", wide.data_ptr(), wide.stride(0), m_rows, out_w[layer].blob.data_ptr(), 0,
+                             h.data_ptr(), hidden, ffn + hidden, GROUP, 0, stream)
 
             graph = graph_of(one_pass_two)
             ms = time_launches(lambda _: graph.replay(), passes, warmup)

@@ -369,6 +369,11 @@ int gq_gemv_sequence_ws_f16(const gq_gemv_desc *descs, const gq_gemv_desc *descs
  *                               pipelined MFMA kernel of gq_gemm_f16 with the blob as its weight source
  *                               (every input feature brings its own scale and bias to the expansion).
  *                               Either way the result is within the tolerance of the fused paths.
+ *   gq_linear_knp_strided_f16   gq_linear_knp_act_f16 at decode batches (m_rows <= 16) for an x whose rows are
+ *                               `x_row_stride` elements apart (>= k_in, a multiple of 8: every row 16-byte
+ *                               aligned): a column slice of a wider matrix, read where it lies (see
+ *                               gq_linear_p_strided_f16).  The same kernel and results as on a gathered x.
+ *                               m_rows > 16: GQ_ERR_UNSUPPORTED; x_row_stride < k_in: GQ_ERR_BAD_SHAPE.
  */
 int64_t gq_gemv_kn_prepacked_bytes(int64_t n_out, int64_t k_in, int64_t group_size);
 int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob,
@@ -376,6 +381,9 @@ int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const 
 int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias,
                           uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation,
                           void *stream);
+int gq_linear_knp_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m_rows, const void *blob,
+                              const uint16_t *out_bias, uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size,
+                              int32_t activation, void *stream);
 
 /*
  * Device-side compress for binary16 input: bit-identical packed/scale/bias to

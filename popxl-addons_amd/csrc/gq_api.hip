@@ -426,22 +426,45 @@ int gq_gemv_kn_prepack_f16(const uint16_t *packed, const uint16_t *scale, const 
   return gq::launch_gemv_kn_prepack(packed, scale, bias, blob, n_out, k_in, (hipStream_t)stream);
 }
 
-int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y,
-                          int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation, void *stream) {
+// argument checks shared by the two entry points on the kn streaming layout; 1 = proceed
+static int check_linear_knp_args(const char *who, const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias,
+                                 uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation) {
   if (m_rows < 0 || n_out < 0 || k_in < 0)
-    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_knp_act_f16: negative size (m_rows=%lld n_out=%lld k_in=%lld)", (long long)m_rows,
+    return gq::fail(GQ_ERR_BAD_SHAPE, "%s: negative size (m_rows=%lld n_out=%lld k_in=%lld)", who, (long long)m_rows,
                     (long long)n_out, (long long)k_in);
   if (activation < GQ_ACT_NONE || activation > GQ_ACT_GELU_TANH)
-    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: unknown activation %d", (int)activation);
+    return gq::fail(GQ_ERR_UNSUPPORTED, "%s: unknown activation %d", who, (int)activation);
   if (m_rows == 0 || n_out == 0) return GQ_OK;
   if (!gq::gemv_kn_prepack_shape_ok(n_out, k_in, group_size))
     return gq::fail(GQ_ERR_UNSUPPORTED,
-                    "gq_linear_knp_act_f16: the kn streaming layout needs group_size 64, n_out %% 64 == 0 and k_in %% 512 == 0 (got "
-                    "group_size=%lld n_out=%lld k_in=%lld)", (long long)group_size, (long long)n_out, (long long)k_in);
-  if (!x || !blob || !y) return gq::fail(GQ_ERR_NULL_POINTER, "gq_linear_knp_act_f16: x, blob and y must not be NULL");
+                    "%s: the kn streaming layout needs group_size 64, n_out %% 64 == 0 and k_in %% 512 == 0 (got "
+                    "group_size=%lld n_out=%lld k_in=%lld)", who, (long long)group_size, (long long)n_out, (long long)k_in);
+  if (!x || !blob || !y) return gq::fail(GQ_ERR_NULL_POINTER, "%s: x, blob and y must not be NULL", who);
   if (gq::misaligned(x, 16) || gq::misaligned(blob, 16) || gq::misaligned(y, 8) || gq::misaligned(out_bias, 2))
-    return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_knp_act_f16: x and blob must be 16-byte aligned, y 8-byte, out_bias 2-byte");
-  if (m_rows > (int64_t)1 << 30) return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_act_f16: m_rows exceeds 2^30");
+    return gq::fail(GQ_ERR_MISALIGNED, "%s: x and blob must be 16-byte aligned, y 8-byte, out_bias 2-byte", who);
+  if (m_rows > (int64_t)1 << 30) return gq::fail(GQ_ERR_UNSUPPORTED, "%s: m_rows exceeds 2^30", who);
+  return 1;
+}
+
+int gq_linear_knp_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m_rows, const void *blob, const uint16_t *out_bias,
+                              uint16_t *y, int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation, void *stream) {
+  const int rc = check_linear_knp_args("gq_linear_knp_strided_f16", x, m_rows, blob, out_bias, y, n_out, k_in, group_size, activation);
+  if (rc <= 0) return rc;
+  if (x_row_stride < k_in)
+    return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_knp_strided_f16: x_row_stride=%lld is less than k_in=%lld", (long long)x_row_stride,
+                    (long long)k_in);
+  if (x_row_stride % 8 != 0)
+    return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_knp_strided_f16: every row of x must be 16-byte aligned (x_row_stride %% 8 == 0)");
+  if (m_rows > 16)
+    return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_strided_f16: m_rows=%lld; rows of x apart are taken up to 16 rows "
+                    "(gather x, or call per 16 rows)", (long long)m_rows);
+  return gq::launch_gemv_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream, x_row_stride);
+}
+
+int gq_linear_knp_act_f16(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y,
+                          int64_t n_out, int64_t k_in, int64_t group_size, int32_t activation, void *stream) {
+  const int args_rc = check_linear_knp_args("gq_linear_knp_act_f16", x, m_rows, blob, out_bias, y, n_out, k_in, group_size, activation);
+  if (args_rc <= 0) return args_rc;
   if (m_rows <= 16) return gq::launch_gemv_knp(x, m_rows, blob, out_bias, y, n_out, k_in, (int)activation, (hipStream_t)stream);
   // 17 to 32 rows: two passes of the decode kernel over 16 rows each are faster than the prefill kernel's
   // mostly empty tiles (as for the other layout)

@@ -104,7 +104,7 @@ int64_t gemv_kn_prepacked_bytes(int64_t n_out, int64_t k_in);
 int launch_gemv_kn_prepack(const uint16_t *packed, const uint16_t *scale, const uint16_t *bias, void *blob, int64_t n_out,
                            int64_t k_in, hipStream_t stream);
 int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
-                    int64_t k_in, int act, hipStream_t stream);
+                    int64_t k_in, int act, hipStream_t stream, int64_t ldx = 0);
 int launch_gemm_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
                     int64_t k_in, int act, hipStream_t stream);
 int launch_compress(const uint16_t *t, uint16_t *packed, uint16_t *scale, uint16_t *bias, int32_t *flag,

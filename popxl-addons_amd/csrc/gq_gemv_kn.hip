@@ -93,7 +93,7 @@ template <int R, int XM>
 __global__ __launch_bounds__(kKnWaves * 64) void gemv_knp_kernel(const half_t *__restrict__ x, int m_rows,
                                                                 const char *__restrict__ blob,
                                                                 const half_t *__restrict__ out_bias, half_t *__restrict__ y,
-                                                                int n_out, int k_in, int act) {
+                                                                int n_out, int k_in, int act, int ldx) {
   constexpr int kRegion = knp_region_bytes(R, XM);
   constexpr int kPerGroup = 4 / R;  // workgroups that share a group of 64 outputs
   extern __shared__ __attribute__((aligned(16))) char knp_lds[];
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kKnWaves * 64) void gemv_knp_kernel(const half_t *_
     k.bv = *reinterpret_cast<const uint4_t *>(u + 17408);
 #pragma unroll
     for (int m = 0; m < XM; ++m)
-      k.xq[m] = *reinterpret_cast<const uint4_t *>(x_lane + ((int64_t)min(m, m_rows - 1) * k_in + c * 512) * 2);
+      k.xq[m] = *reinterpret_cast<const uint4_t *>(x_lane + ((int64_t)min(m, m_rows - 1) * ldx + c * 512) * 2);  // (rows of x: ldx elements apart)
 #pragma unroll
     for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -296,9 +296,10 @@ int launch_gemv_kn_prepack(const uint16_t *packed, const uint16_t *scale, const 
   return check_launch("kn_prepack_kernel");
 }
 
-// One GEMV on a weight in the kn streaming layout (m_rows <= 16; the caller has checked the shape).
+// One GEMV on a weight in the kn streaming layout (m_rows <= 16; the caller has checked the shape).  ldx: elements
+// from a row of x to the next (0: k_in; a multiple of 8).
 int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const uint16_t *out_bias, uint16_t *y, int64_t n_out,
-                    int64_t k_in, int act, hipStream_t stream) {
+                    int64_t k_in, int act, hipStream_t stream, int64_t ldx) {
   const int64_t groups = n_out / 64;
   // Row blocks per wave (1, 2 or 4: they share the scaled activations): the choice that moves the
   // fewest bytes per busy compute unit -- the codes once, scales, biases and x once per workgroup
@@ -335,7 +336,8 @@ int launch_gemv_knp(const uint16_t *x, int64_t m_rows, const void *blob, const u
     }                                                                                                         \
     gemv_knp_kernel<R, XM><<<dim3(blocks), dim3(kKnWaves * 64), lds_bytes, stream>>>(                         \
         reinterpret_cast<const half_t *>(x), (int)m_rows, reinterpret_cast<const char *>(blob),               \
-        reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, act); \
+        reinterpret_cast<const half_t *>(out_bias), reinterpret_cast<half_t *>(y), (int)n_out, (int)k_in, act,  \
+        (int)(ldx ? ldx : k_in));                                                                             \
   } while (0)
 #define GQ_KNP_BY_R(XM)                            \
   do {                                             \

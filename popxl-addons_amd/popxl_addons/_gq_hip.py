@@ -55,6 +55,7 @@ EXPORTS = (
     "gq_gemv_kn_prepacked_bytes",
     "gq_gemv_kn_prepack_f16",
     "gq_linear_knp_act_f16",
+    "gq_linear_knp_strided_f16",
     "gq_compress_f16",
     "gq_compress_f32",
 )
@@ -133,6 +134,8 @@ def load():
     lib.gq_gemv_kn_prepack_f16.restype = ctypes.c_int
     lib.gq_linear_knp_act_f16.argtypes = [p, i64, p, p, p, i64, i64, i64, ctypes.c_int32, p]
     lib.gq_linear_knp_act_f16.restype = ctypes.c_int
+    lib.gq_linear_knp_strided_f16.argtypes = [p, i64, i64, p, p, p, i64, i64, i64, ctypes.c_int32, p]
+    lib.gq_linear_knp_strided_f16.restype = ctypes.c_int
     for name in ("gq_compress_f16", "gq_compress_f32"):
         fn = getattr(lib, name)
         fn.argtypes = [p, p, p, p, p, i64, i64, i64, p]
@@ -231,17 +234,24 @@ def prepack_gemv_kn(packed, scale, bias):
 
 def linear_knp(x, weight, out_bias=None, activation=None, y=None):
     """y = act(x @ w + out_bias) for x float16 [m_rows, k_in] on the GPU and a PrepackedWeight in the kn
-    streaming layout (gq_linear_knp_act_f16: the decode kernel up to 16 rows, the MFMA pipeline above)."""
+    streaming layout (gq_linear_knp_act_f16: the decode kernel up to 16 rows, the MFMA pipeline above).
+    A decode batch (up to 16 rows) may be a column slice of a wider matrix -- unit stride along the features,
+    rows a multiple of 8 elements apart: it is read where it lies (gq_linear_knp_strided_f16)."""
     import torch
 
-    assert weight.layout == "kn" and x.is_cuda and x.is_contiguous() and x.shape[-1] == weight.k_in
+    assert weight.layout == "kn" and x.is_cuda and x.dim() == 2 and x.shape[-1] == weight.k_in
     m_rows = x.shape[0]
+    strided = not x.is_contiguous()
+    assert not strided or (x.stride(1) == 1 and x.stride(0) >= weight.k_in and x.stride(0) % 8 == 0 and m_rows <= 16)
     with torch.cuda.device(x.device):
         if y is None:
             y = torch.empty((m_rows, weight.n_out), dtype=torch.float16, device=x.device)
-        call("gq_linear_knp_act_f16", x.data_ptr(), m_rows, weight.blob.data_ptr(), 0 if out_bias is None else out_bias.data_ptr(),
-             y.data_ptr(), weight.n_out, weight.k_in, weight.group_size, activation_code(activation),
-             torch.cuda.current_stream(x.device).cuda_stream)
+        tail = (weight.blob.data_ptr(), 0 if out_bias is None else out_bias.data_ptr(), y.data_ptr(), weight.n_out, weight.k_in,
+                weight.group_size, activation_code(activation), torch.cuda.current_stream(x.device).cuda_stream)
+        if strided:
+            call("gq_linear_knp_strided_f16", x.data_ptr(), x.stride(0), m_rows, *tail)
+        else:
+            call("gq_linear_knp_act_f16", x.data_ptr(), m_rows, *tail)
     return y
 
 

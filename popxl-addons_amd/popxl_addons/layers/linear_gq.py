@@ -129,7 +129,9 @@ class LinearGQ:
         # A decode batch that is a column slice of a wider matrix (part of the output of fused projections, say)
         # is read where it lies, its rows a stride apart; anything else is gathered into a contiguous x.
         x_row_stride = 0
-        if (self.dim == 0 and x.dim() == 2 and not x.is_contiguous() and x.stride(1) == 1 and x.stride(0) >= in_features
+        takes_stride = self.dim == 0 or (self._decode_copy is not None and x.data_ptr() % 16 == 0 and x.dim() == 2
+                                         and x.stride(0) % 8 == 0)
+        if (takes_stride and x.dim() == 2 and not x.is_contiguous() and x.stride(1) == 1 and x.stride(0) >= in_features
                 and 0 < x.shape[0] <= 16):
             x2, x_row_stride = x, x.stride(0)
         else:
@@ -151,7 +153,7 @@ class LinearGQ:
                 act,
             )
             stream = torch.cuda.current_stream(x.device).cuda_stream
-            if x_row_stride:
+            if x_row_stride and self.dim == 0:
                 blob = 0 if self._decode_copy is None else self._decode_copy.blob.data_ptr()
                 _gq_hip.call("gq_linear_p_strided_f16", args[0], x_row_stride, *args[1:5], blob, *args[5:], stream)
             elif self.dim == 0:
@@ -163,7 +165,7 @@ class LinearGQ:
                 _gq_hip.call("gq_linear_p_act_f16", *args[:5], blob, *args[5:], 0 if ws is None else ws.data_ptr(),
                              0 if ws is None else ws.numel(), stream)
             elif self._decode_copy is not None:
-                # groups along the output features, the derived copy is there
+                # groups along the output features, the derived copy is there (x2 contiguous, or rows a stride apart)
                 _gq_hip.linear_knp(x2, self._decode_copy, b, act, y)
             else:
                 # groups along the output features: weight rows are input features

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from gq_testlib import activations, to_dev
+from gq_testlib import activations, assert_bits_equal, to_dev
 from popxl_addons.layers.linear_gq import LinearGQ
 from popxl_addons.ops.group_quantize_decompress import group_quantize_compress_numpy
 from test_gpu_fused import assert_close
@@ -177,6 +177,25 @@ def test_agrees_with_the_kernel_on_the_variables(hip, device, oracle):
     assert_close(y_blob.cpu().numpy(), ref, "blob")
 
 
+@pytest.mark.parametrize("k_in,n_out", [(4096, 4096), (4096, 16384), (16384, 4096), (1536, 320)])
+@pytest.mark.parametrize("m_rows", [1, 4, 8, 16])
+def test_rows_of_x_a_stride_apart(hip, device, oracle, k_in, n_out, m_rows):
+    """gq_linear_knp_strided_f16: x as a column slice of a wider matrix gives the bits of the call on the gathered
+    x (the same kernel reads it where it lies), and the oracle's result."""
+    from popxl_addons._gq_hip import linear_knp
+
+    copy, _, w_dec_t = _weight(oracle, device, k_in, n_out, 11)
+    ob = np.random.default_rng(91).normal(0, 1, (n_out,)).astype(np.float16)
+    wide = to_dev(activations(m_rows, k_in + 264, 90 + m_rows), device)
+    for offset in (0, 136):
+        part = wide[:, offset : offset + k_in]
+        assert not part.is_contiguous() or m_rows == 1
+        y = linear_knp(part, copy, to_dev(ob, device), "relu").cpu().numpy()
+        gathered = linear_knp(part.contiguous(), copy, to_dev(ob, device), "relu").cpu().numpy()
+        assert_bits_equal(y, gathered, (k_in, n_out, m_rows, offset))
+        assert_close(y, oracle.np_linear(part.cpu().numpy(), w_dec_t, ob, "relu"), (k_in, n_out, m_rows, offset))
+
+
 def test_rejected_arguments(hip, device):
     from popxl_addons._gq_hip import GQ_ERR_MISALIGNED, GQ_ERR_UNSUPPORTED, GQHipError
 
@@ -222,6 +241,10 @@ def test_layer_serves_decode_batches_from_the_copy(hip, device, oracle, dim):
             ref = oracle.np_linear(x.reshape(-1, 1024), w_dec_t, v.bias.data.cpu().numpy(), "relu").reshape(*batch, 1024)
             assert_close(y, ref, (round_, batch))
             refs.append(ref)
+        # a decode batch that is a column slice of a wider matrix is read where it lies: the gathered call's bits
+        wide = to_dev(np.random.default_rng(60 + round_).normal(0, 1, (5, 1024 + 512)).astype(np.float16), device)
+        part = wide[:, 256 : 256 + 1024]
+        assert_bits_equal(layer(part).cpu().numpy(), layer(part.contiguous()).cpu().numpy(), (round_, "slice"))
 
 
 @pytest.mark.parametrize("m_rows", [1, 8])

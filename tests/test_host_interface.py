@@ -85,6 +85,15 @@ def test_abi_version_and_error_text_without_gpu():
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_p_strided_f16", 16, 1024, 4, 16, 0, 16, 16, 0, 16, 8, 512, 64, 0, None)  # scale NULL, the others not
     assert e.value.code == _gq_hip.GQ_ERR_NULL_POINTER
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_knp_strided_f16", 16, 1024, 17, 16, 0, 16, 64, 512, 64, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_UNSUPPORTED and "16 rows" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_knp_strided_f16", 16, 1028, 4, 16, 0, 16, 64, 512, 64, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_MISALIGNED and "x_row_stride" in str(e.value)
+    with pytest.raises(_gq_hip.GQHipError) as e:
+        _gq_hip.call("gq_linear_knp_strided_f16", 16, 256, 4, 16, 0, 16, 64, 512, 64, 0, None)
+    assert e.value.code == _gq_hip.GQ_ERR_BAD_SHAPE
     # the [k_in, n_out] layout: its own argument rules and the workspace contract
     with pytest.raises(_gq_hip.GQHipError) as e:
         _gq_hip.call("gq_linear_kn_act_f16", 16, 1, 16, 16, 16, 0, 16, 96, 64, 64, 0, None, 0, None)  # 96 % 64 != 0
