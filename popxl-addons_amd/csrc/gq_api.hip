@@ -214,6 +214,7 @@ int gq_linear_p_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m_r
   if (x_row_stride < k_in)
     return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_p_strided_f16: x_row_stride=%lld is less than k_in=%lld", (long long)x_row_stride,
                     (long long)k_in);
+  if (x_row_stride > (int64_t)1 << 30) return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_p_strided_f16: x_row_stride exceeds 2^30");
   if (m_rows > 16)
     return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_p_strided_f16: m_rows=%lld; rows of x apart are taken up to 16 rows "
                     "(gather x, or call per 16 rows)", (long long)m_rows);
@@ -453,6 +454,7 @@ int gq_linear_knp_strided_f16(const uint16_t *x, int64_t x_row_stride, int64_t m
   if (x_row_stride < k_in)
     return gq::fail(GQ_ERR_BAD_SHAPE, "gq_linear_knp_strided_f16: x_row_stride=%lld is less than k_in=%lld", (long long)x_row_stride,
                     (long long)k_in);
+  if (x_row_stride > (int64_t)1 << 30) return gq::fail(GQ_ERR_UNSUPPORTED, "gq_linear_knp_strided_f16: x_row_stride exceeds 2^30");
   if (x_row_stride % 8 != 0)
     return gq::fail(GQ_ERR_MISALIGNED, "gq_linear_knp_strided_f16: every row of x must be 16-byte aligned (x_row_stride %% 8 == 0)");
   if (m_rows > 16)
