@@ -163,6 +163,56 @@ def test_rows_of_x_a_stride_apart(hip, device, oracle, n_out, k_in, m_rows):
     assert e.value.code == GQ_ERR_MISALIGNED
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_decode_problems_through_every_route(hip, device, oracle, seed):
+    """Seeded random problems at decode batches: shapes that fill or do not fill chunks of 512 features and groups of
+    8 row blocks, group sizes 32 / 64 / 128, one to sixteen rows, x gathered or a column slice (aligned or not), with
+    the copy (where one exists), without it, and the copy alone: whichever kernel the routing picks, the oracle's
+    result; the copy and the variables agree bit for bit wherever both run the same kernel (an aligned x)."""
+    rng = np.random.default_rng(1000 + seed)
+    gs = int(rng.choice([32, 64, 64, 64, 128]))
+    k_in = int(rng.choice([128, 256, 512, 640, 1024, 1536, 2048, 4096])) if seed % 3 else int(rng.choice([512, 1024, 2048]))
+    k_in = max(k_in, gs)
+    n_out = int(rng.choice([16, 40, 128, 1000, 3336, 4096])) if seed % 3 else int(rng.choice([26624, 28680, 33000]))
+    m_rows = int(rng.integers(1, 17))
+    offset = int(rng.choice([0, 0, 8, 24, 3]))
+    pad = int(rng.choice([0, 64, 200]))
+    w = (rng.normal(0, 0.02, (n_out, k_in)) * np.exp(rng.normal(0, 0.5, (n_out, 1)))).astype(np.float16)
+    packed, scale, bias = group_quantize_compress_numpy(w, gs)
+    w_dec = oracle.np_decompress(packed, scale, bias)
+    dev = tuple(to_dev(a, device) for a in (packed, scale, bias))
+    has_copy = gs == 64 and k_in % 512 == 0
+    copy = hip.prepack_gemv(*dev) if has_copy else None
+    wide = activations(m_rows, k_in + offset + pad, 2000 + seed)
+    x = np.ascontiguousarray(wide[:, offset : offset + k_in])
+    ob = rng.normal(0, 1, (n_out,)).astype(np.float16) if seed % 2 else None
+    act, name = [(0, None), (1, "relu"), (2, "gelu_tanh")][seed % 3]
+    ref = oracle.np_linear(x, w_dec, ob, name)
+    wd, od = to_dev(wide, device), None if ob is None else to_dev(ob, device)
+    stream = torch.cuda.current_stream().cuda_stream
+    aligned = offset % 8 == 0 and (k_in + offset + pad) % 8 == 0
+
+    def strided(variables, blob):
+        y = torch.full((m_rows, n_out), float("nan"), dtype=torch.float16, device=device)
+        v = [t.data_ptr() for t in dev] if variables else [0, 0, 0]
+        hip.call("gq_linear_p_strided_f16", wd.data_ptr() + 2 * offset, k_in + offset + pad, m_rows, *v,
+                 copy.blob.data_ptr() if blob else 0, 0 if od is None else od.data_ptr(), y.data_ptr(), n_out, k_in, gs, act, stream)
+        torch.cuda.synchronize()
+        return y.cpu().numpy()
+
+    what = (seed, gs, n_out, k_in, m_rows, offset, pad)
+    from_variables = strided(True, False)
+    assert_close(from_variables, ref, what)
+    assert_close(_run(hip, device, x, dev, None, ob, n_out, k_in, act) if gs == 64 else from_variables, ref, what)
+    if has_copy:
+        with_copy = strided(True, True)
+        assert_close(with_copy, ref, what)
+        if aligned:
+            assert_bits_equal(with_copy, from_variables, what)
+            assert_bits_equal(strided(False, True), from_variables, what)
+            assert_bits_equal(_run(hip, device, x, dev, copy.blob, ob, n_out, k_in, act), from_variables, what)
+
+
 def test_layer_reads_a_column_slice_where_it_lies(hip, device, oracle):
     """LinearGQ(dim=0).build on a decode batch that is a column slice of a wider matrix: no gather, the result of the
     gathered call bit for bit; a slice of more than 16 rows is gathered as before."""
