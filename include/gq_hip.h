@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define GQ_ABI_VERSION 3
+#define GQ_ABI_VERSION 4
 
 #define GQ_OK 0
 #define GQ_ERR_NULL_POINTER (-1) /* a required pointer is NULL */

@@ -10,7 +10,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 _DEFAULT_LIB = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libgq_hip.so")
 
-GQ_ABI_VERSION = 3
+GQ_ABI_VERSION = 4
 GQ_ERR_NULL_POINTER = -1
 GQ_ERR_BAD_SHAPE = -2
 GQ_ERR_MISALIGNED = -3
