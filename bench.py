@@ -901,7 +901,7 @@ def main():
             cpu["legs"] = cpu_baseline_legs()
             for leg in cpu["legs"]:
                 log(f"  cpu: {leg['workload']}: {leg['seconds']:.3f} s, {leg['value']:.3f} {leg['unit']}")
-    if args.only == "all":
+    if args.only in ("all", "decompress"):
         # the same weight with the result transposed (dim=0 of the operator)
         outs_t = [torch.empty((16384, 4096), dtype=torch.float16, device=device) for _ in dec["sets"]]
 
